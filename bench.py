@@ -1,0 +1,315 @@
+#!/usr/bin/env python3
+"""Benchmark of the device kernel library on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic input, with
+all inputs already resident in HBM when the timed region starts.  The headline
+workload is the LayerNorm configuration of BASELINE.json (configs[1]:
+fp32 (32,128,768), eps 1e-5); the other configurations (add, fp16 LayerNorm,
+fused MHA at three shapes, the BERT-base layer) are measured in the same run
+and reported under "kernels" in the same JSON line, each against the roofline
+that bounds it.
+
+Timing: K launches are enqueued back to back on one stream between two HIP
+events recorded on that same stream (captured into one hipGraph so the host
+launch cost does not throttle microsecond kernels).  Memory-bound kernels rotate
+through enough distinct buffer sets (> 256 MiB in total) that no launch finds
+its operands in the Infinity Cache left by an earlier one; the cache-resident
+("warm") figure is reported next to it.
+
+The CPU baseline times the oracle (a plain C port of the reference semantics)
+on the host cores for a bounded sample; it is a reported baseline, not the
+target.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+MALL_BYTES = 256 << 20
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="enqueue launches directly instead of through a hipGraph")
+    ap.add_argument("--only", type=str, default="", help="comma list of kernels to run besides the headline")
+    return ap.parse_args()
+
+
+class Timer:
+    """Times `steps` launches of fn(i) on the current torch stream."""
+
+    def __init__(self, torch, use_graph: bool):
+        self.torch = torch
+        self.use_graph = use_graph
+
+    def run(self, fn, steps: int, warmup: int) -> float:
+        """Returns elapsed milliseconds for exactly `steps` launches."""
+        torch = self.torch
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            for i in range(warmup):
+                fn(i)
+            stream.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            graph = None
+            if self.use_graph:
+                try:
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, stream=stream):
+                        for i in range(steps):
+                            fn(i)
+                    graph.replay()  # untimed first replay (upload)
+                    stream.synchronize()
+                except Exception as exc:  # capture unsupported for this op: time direct launches
+                    print(f"[bench] graph capture failed ({exc}); timing direct launches", file=sys.stderr)
+                    graph = None
+                    torch.cuda.synchronize()
+            torch.cuda.synchronize()
+            e0.record(stream)
+            if graph is not None:
+                graph.replay()
+            else:
+                for i in range(steps):
+                    fn(i)
+            e1.record(stream)
+            e1.synchronize()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1)
+
+
+def rotating_sets(bytes_per_set: int) -> int:
+    """Number of buffer sets whose total footprint exceeds the Infinity Cache."""
+    return max(2, (MALL_BYTES + bytes_per_set - 1) // bytes_per_set + 2)
+
+
+def hbm_entry(name, workload, dtype, bytes_per_launch, ms, steps, warm_ms=None):
+    us = ms * 1e3 / steps
+    gbs = bytes_per_launch / us / 1e3
+    e = {"name": name, "workload": workload, "dtype": dtype, "metric": "GB/s", "value": round(gbs, 1),
+         "us_per_launch": round(us, 3),
+         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+         "algorithmic_bytes": bytes_per_launch}
+    if warm_ms is not None:
+        wus = warm_ms * 1e3 / steps
+        e["cache_resident"] = {"us_per_launch": round(wus, 3), "GB/s": round(bytes_per_launch / wus / 1e3, 1)}
+    return e
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus must be 1 (multi-GPU runs are not part of it)",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import __graft_entry__ as ge
+
+    pkg = ge.load_package()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    if not pkg.is_built():
+        ge.build()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = pkg.ops()
+    timer = Timer(torch, use_graph=not args.no_graph)
+    K, W = args.steps, args.warmup
+    only = set(filter(None, args.only.split(",")))
+
+    def want(name):
+        return not only or name in only
+
+    def check():
+        msg = lib.mgpuOpsTakeLastError()
+        if msg is not None:
+            raise RuntimeError(msg.decode())
+
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(20241)
+    kernels = []
+
+    # ---------------- headline: LayerNorm fp32 (32,128,768) -------------------
+    m, n = 32 * 128, 768
+    ln_bytes = 2 * m * n * 4 + 2 * n * 4
+    nsets = rotating_sets(2 * m * n * 4)
+    xs = [torch.randn((m, n), device=dev, generator=gen) for _ in range(nsets)]
+    ys = [torch.empty((m, n), device=dev) for _ in range(nsets)]
+    gamma = 1 + 0.02 * torch.randn(n, device=dev, generator=gen)
+    beta = 0.02 * torch.randn(n, device=dev, generator=gen)
+
+    def ln32(i, xs=xs, ys=ys):
+        s = torch.cuda.current_stream().cuda_stream
+        lib.mgpuLayerNormF32(xs[i % len(xs)].data_ptr(), gamma.data_ptr(), beta.data_ptr(),
+                             ys[i % len(ys)].data_ptr(), 1e-5, m, n, s)
+
+    ms_cold = timer.run(ln32, K, W)
+    check()
+    ms_warm = timer.run(lambda i: ln32(0), K, W)
+    check()
+    headline = hbm_entry("layernorm_f32", "LayerNorm fp32 (32,128,768) eps=1e-5 [configs[1]]", "f32",
+                         ln_bytes, ms_cold, K, ms_warm)
+    del xs, ys
+
+    # ---------------- LayerNorm fp16 ------------------------------------------
+    if want("layernorm_f16"):
+        nsets = rotating_sets(2 * m * n * 2)
+        xh = [torch.randn((m, n), device=dev, generator=gen).half() for _ in range(nsets)]
+        yh = [torch.empty((m, n), device=dev, dtype=torch.float16) for _ in range(nsets)]
+        gh, bh = gamma.half(), beta.half()
+
+        def ln16(i):
+            s = torch.cuda.current_stream().cuda_stream
+            lib.mgpuLayerNormF16(xh[i % nsets].data_ptr(), gh.data_ptr(), bh.data_ptr(),
+                                 yh[i % nsets].data_ptr(), 1e-5, m, n, s)
+
+        ms = timer.run(ln16, K, W)
+        msw = timer.run(lambda i: ln16(0), K, W)
+        check()
+        kernels.append(hbm_entry("layernorm_f16", "LayerNorm fp16 (32,128,768)", "f16",
+                                 2 * m * n * 2 + 2 * n * 2, ms, K, msw))
+        del xh, yh
+
+    # ---------------- add fp32 (3,640,640) -------------------------------------
+    if want("add_f32"):
+        ne = 3 * 640 * 640
+        nsets = rotating_sets(3 * ne * 4)
+        aa = [torch.rand(ne, device=dev, generator=gen) * 2 - 1 for _ in range(nsets)]
+        bb = [torch.rand(ne, device=dev, generator=gen) * 2 - 1 for _ in range(nsets)]
+        cc = [torch.empty(ne, device=dev) for _ in range(nsets)]
+
+        def add(i):
+            s = torch.cuda.current_stream().cuda_stream
+            j = i % nsets
+            lib.mgpuAddF32(aa[j].data_ptr(), bb[j].data_ptr(), cc[j].data_ptr(), ne, s)
+
+        ms = timer.run(add, K, W)
+        msw = timer.run(lambda i: add(0), K, W)
+        check()
+        kernels.append(hbm_entry("add_f32", "add fp32 (3,640,640) [configs[0]]", "f32", 3 * ne * 4, ms, K, msw))
+        del aa, bb, cc
+
+    # ---------------- fused MHA -------------------------------------------------
+    def fmha_case(name, workload, B, S, H, masked):
+        D = 64
+        qkv = (torch.randn((B, S, 3, H, D), device=dev, generator=gen) / 8).half()
+        out = torch.empty((B, S, H * D), device=dev, dtype=torch.float16)
+        lens = None
+        flop = 4.0 * B * H * S * S * D
+        if masked:
+            lens_cpu = torch.randint(256, 513, (B,), generator=torch.Generator().manual_seed(20244), dtype=torch.int32)
+            lens = lens_cpu.to(dev)
+            flop_valid = 4.0 * H * D * S * float(lens_cpu.sum())
+        else:
+            flop_valid = flop
+
+        def run(i):
+            s = torch.cuda.current_stream().cuda_stream
+            lib.mgpuFusedMHAF16(qkv.data_ptr(), lens.data_ptr() if lens is not None else None,
+                                out.data_ptr(), B, S, H, D, 0.125, 0, s)
+
+        steps = max(20, K // 4)
+        ms = timer.run(run, steps, max(3, W // 4))
+        check()
+        us = ms * 1e3 / steps
+        tf = flop_valid / us / 1e6
+        nbytes = qkv.numel() * 2 + out.numel() * 2 + (4 * B if masked else 0)
+        entry = {"name": name, "workload": workload, "dtype": "f16", "metric": "TFLOP/s", "value": round(tf, 1),
+                 "us_per_launch": round(us, 3),
+                 "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                              "unit": "TFLOP/s", "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+                 "algorithmic_flop": flop_valid, "algorithmic_bytes": nbytes,
+                 "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        if masked:
+            entry["dense_flop"] = flop
+        kernels.append(entry)
+
+    if want("fmha_b32_s128"):
+        fmha_case("fmha_b32_s128", "fused MHA fp16 b32 s128 h12 d64 [configs[2]]", 32, 128, 12, False)
+    if want("fmha_b8_s512_masked"):
+        fmha_case("fmha_b8_s512_masked", "fused MHA fp16 b8 s512 h16 d64, key lengths U[256,512] [configs[3]]",
+                  8, 512, 16, True)
+    if want("fmha_b32_s512"):
+        fmha_case("fmha_b32_s512", "fused MHA fp16 b32 s512 h12 d64 [roofline target shape]", 32, 512, 12, False)
+
+    # ---------------- BERT-base encoder layer ----------------------------------
+    if want("bert_layer"):
+        B, S, d, ffn, H = 32, 128, 768, 3072, 12
+
+        def w(*shape, s=0.02):
+            return (s * torch.randn(shape, device=dev, generator=gen)).half()
+
+        x = torch.randn((B, S, d), device=dev, generator=gen).half()
+        P = [w(d, 3 * d), w(3 * d), w(d, d), w(d), (1 + w(d).float()).half(), w(d), w(d, ffn), w(ffn),
+             w(ffn, d), w(d), (1 + w(d).float()).half(), w(d)]
+        out = torch.empty_like(x)
+
+        def layer(i):
+            s = torch.cuda.current_stream().cuda_stream
+            lib.mgpuBertEncoderLayerF16(x.data_ptr(), *[p.data_ptr() for p in P], None, out.data_ptr(),
+                                        B, S, d, ffn, H, 1e-5, s)
+
+        steps = max(10, K // 10)
+        ms = Timer(torch, use_graph=False).run(layer, steps, 3)
+        check()
+        us = ms * 1e3 / steps
+        flop = 2.0 * B * S * d * (3 * d + d + ffn + ffn) + 4.0 * B * H * S * S * 64
+        kernels.append({"name": "bert_layer", "workload": "BERT-base encoder layer fp16 (32,128,768) [configs[4]]",
+                        "dtype": "f16", "metric": "us", "value": round(us, 1), "higher_is_better": False,
+                        "roofline": {"bound": "mfma", "achieved": round(flop / us / 1e6, 1),
+                                     "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                     "frac": round(flop / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+                        "algorithmic_flop": flop})
+
+    # ---------------- CPU baseline: the oracle on the host cores ---------------
+    cpu = None
+    if not args.no_cpu:
+        oracle = ge.load_oracle()
+        rng = np.random.default_rng(20241)
+        x = rng.standard_normal((m, n)).astype(np.float32)
+        g = (1 + 0.02 * rng.standard_normal(n)).astype(np.float32)
+        b = (0.02 * rng.standard_normal(n)).astype(np.float32)
+        threads = oracle.num_threads()
+        oracle.layernorm(x, g, b)
+        reps, t0 = 0, time.perf_counter()
+        while reps < 2000 and time.perf_counter() - t0 < 10.0:
+            oracle.layernorm(x, g, b)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        cpu = {"value": round(ln_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+               "sample": f"{reps} passes of LayerNorm fp32 (32,128,768) through oracle_layernorm "
+                         f"(fp64 arithmetic, OpenMP, {threads} threads), {dt * 1e6:.0f} us per pass"}
+
+    result = {
+        "metric": "LayerNorm GB/s (fp32 (32,128,768)); fMHA TFLOP/s and BERT-base layer us under 'kernels'",
+        "value": headline["value"], "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_cold / K, 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": headline["workload"], "rows": m, "cols": n, "eps": 1e-5,
+                   "launch_mode": "direct" if args.no_graph else "hipGraph of K launches",
+                   "buffer_sets": rotating_sets(2 * m * n * 4)},
+        "roofline": headline["roofline"], "cache_resident": headline.get("cache_resident"),
+        "cpu_baseline": cpu, "kernels": kernels,
+        "device": torch.cuda.get_device_name(0),
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

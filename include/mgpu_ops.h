@@ -1,0 +1,155 @@
+/*
+ * mgpu_ops.h - C ABI of the device kernel library (libmgpu_hip_ops.so) for one
+ * MI355X: LayerNorm, fused multi-head attention, elementwise add, casts,
+ * GEMM with epilogue, and the transformer layers composed from them.
+ *
+ * Drop-in for the kernel library the reference's compiled models call by
+ * symbol name (include/multi-device-model-compiler/Kernels/GPU/Ops.h:15-74,
+ * Utils.h:6-8).  The reference exports only mgpuMatmul / mgpuConv2d /
+ * mgpuPool2d / mgpuLLMDecodingContextLayer as `extern "C"` (Ops.h:22-49); its
+ * LayerNorm, matmulEx, cast and QKV-transpose entry points are C++ templates
+ * instantiated for `half` only, and it has no standalone entry point for
+ * attention, fp32 LayerNorm or add (attention is reachable only through
+ * lib/Kernels/GPU/LLM.cu:79-81, add only as a compiler-generated kernel).  This
+ * header gives every one of them a plain C name with the element type in the
+ * suffix; the C++ header Kernels/GPU/Ops.h of this build keeps the reference's
+ * template names as thin wrappers over these.
+ *
+ * Conventions kept from the reference:
+ *  - all data pointers are DEVICE pointers owned by the caller; the functions
+ *    only enqueue work on `stream` (always the last argument) and return;
+ *  - every function returns void.  The reference prints and throws
+ *    std::logic_error on failure (lib/Kernels/GPU/Ops.cu:21-41); a C caller
+ *    cannot catch that, so the extern "C" layer prints the message to stderr,
+ *    records it, and returns without launching: query it with
+ *    mgpuOpsTakeLastError().  The C++ template wrappers do throw.
+ *  - 16-bit element types are passed as `const void *` holding IEEE binary16
+ *    ("F16") or bfloat16 ("BF16") values.
+ */
+#ifndef MGPU_OPS_H_
+#define MGPU_OPS_H_
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *mgpuStream_t; /* hipStream_t */
+
+/* ---- library lifetime (Ops.h:15-18; Ops.cu:43-55; LLM.cu:14-24) ------- */
+/* C names for gpuOpsInit()/gpuOpsDeinit(): create the hipBLASLt handle and its
+ * workspace, the side stream + event the layer entry points use for casts. */
+void mgpuOpsInit(void);
+void mgpuOpsDeinit(void);
+/* Returns the message of the most recent failure on the calling thread, or
+ * NULL; the message stays valid until the next failing call.  Clears it. */
+const char *mgpuOpsTakeLastError(void);
+
+/* ---- elementwise add -------------------------------------------------- */
+/* c[i] = a[i] + b[i], i < n, IEEE binary32, bit exact.  Replaces the kernel
+ * the reference's pipeline generates for onnx.Add and launches through
+ * mgpuLaunchKernel (lib/Pipelines/MLIRToGPU.cpp:94-135,
+ * lib/Dialect/Device/IR/GPUOffloadingAttr.cpp:283-304); CPU twin
+ * examples/add.ll:42-66. */
+void mgpuAddF32(const float *a, const float *b, float *c, int64_t n, mgpuStream_t stream);
+
+/* ---- LayerNorm -------------------------------------------------------- */
+/* output[r,:] = (input[r,:] - mean_r) * rsqrt(var_r + eps) * gamma + beta for
+ * m rows of n elements (biased variance, statistics in fp32).
+ * Replaces mgpuLayerNorm<T> (Ops.h:57-61; lib/Kernels/GPU/LayerNorm.cu:410-436,
+ * kernel :138-260).  `scale` of the reference signature (int8 quantisation,
+ * unused on this path) is dropped.  gamma and beta must be non-null.  Unlike
+ * the reference any n >= 1 is accepted (the reference needs n even). */
+void mgpuLayerNormF32(const float *input, const float *gamma, const float *beta, float *output,
+                      float eps, int32_t m, int32_t n, mgpuStream_t stream);
+void mgpuLayerNormF16(const void *input, const void *gamma, const void *beta, void *output,
+                      float eps, int32_t m, int32_t n, mgpuStream_t stream);
+void mgpuLayerNormBF16(const void *input, const void *gamma, const void *beta, void *output,
+                       float eps, int32_t m, int32_t n, mgpuStream_t stream);
+
+/* output = round(fp32(input) + fp32(residual)); normed_output = LayerNorm(output)
+ * with the statistics taken from the un-rounded sums.  Replaces
+ * mgpuAddResidualPreLayerNorm<T> (Ops.h:63-68; LayerNorm.cu:438-466). */
+void mgpuAddResidualPreLayerNormF32(const float *input, const float *residual, const float *gamma,
+                                    const float *beta, float *output, float *normed_output,
+                                    float eps, int32_t m, int32_t n, mgpuStream_t stream);
+void mgpuAddResidualPreLayerNormF16(const void *input, const void *residual, const void *gamma,
+                                    const void *beta, void *output, void *normed_output,
+                                    float eps, int32_t m, int32_t n, mgpuStream_t stream);
+void mgpuAddResidualPreLayerNormBF16(const void *input, const void *residual, const void *gamma,
+                                     const void *beta, void *output, void *normed_output,
+                                     float eps, int32_t m, int32_t n, mgpuStream_t stream);
+
+/* ---- fused multi-head attention -------------------------------------- */
+/* out[b,i,h,:] = sum_j softmax_j(scale * <q[b,i,h,:], k[b,j,h,:]>) v[b,j,h,:]
+ * qkv: packed [B, S, 3, H, D]; out: [B, S, H*D]; D must be 64.
+ * seqlens: NULL, or B int32 valid key counts (keys j >= seqlens[b] are masked
+ * out; all S query rows are produced).  causal != 0 also masks j > i.
+ * No score matrix is written to memory.
+ * Replaces FusedMHARunnerFP16v2::setup_causal_masked_fmha + run_causal_masked_fmha
+ * (3rdparty/trt_fused_multihead_attention/qkvToContext.cu:162-199,306-315) as
+ * called at lib/Kernels/GPU/LLM.cu:79-81.  The reference takes b+1 prefix sums
+ * (fused_multihead_attention_v2.h:63-64); this takes per-sequence lengths. */
+void mgpuFusedMHAF16(const void *qkv, const int32_t *seqlens, void *out, int32_t B, int32_t S,
+                     int32_t H, int32_t D, float scale, int32_t causal, mgpuStream_t stream);
+void mgpuFusedMHABF16(const void *qkv, const int32_t *seqlens, void *out, int32_t B, int32_t S,
+                      int32_t H, int32_t D, float scale, int32_t causal, mgpuStream_t stream);
+
+/* ---- casts (Utils.h:6-8; lib/Kernels/GPU/Utils.cu:85-103) ------------- */
+void mgpuCastF32ToF16(void *dst, const float *src, size_t size, mgpuStream_t stream);
+void mgpuCastF16ToF32(float *dst, const void *src, size_t size, mgpuStream_t stream);
+
+/* ---- QKV bias + transpose (Ops.h:70-74; Transpose.cu:70-84) ----------- */
+/* QKV [token,3,H,D] += bias[3,H,D] in place; q/k/v_buf receive [B,H,S,D]. */
+void mgpuAddFusedQKVBiasTransposeF16(void *q_buf, void *k_buf, void *v_buf, void *QKV,
+                                     const void *qkv_bias, int32_t batch_size, int32_t seq_len,
+                                     int32_t token_num, int32_t head_num, int32_t size_per_head,
+                                     mgpuStream_t stream);
+
+/* ---- GEMM ------------------------------------------------------------- */
+/* output[M,N] = input[M,K] . weight[K,N] + bias[N], fp32, row major
+ * (Ops.h:23-25; lib/Kernels/GPU/Ops.cu:57-120). */
+void mgpuMatmul(float *input, float *weight, float *bias, float *output, int64_t M, int64_t N,
+                int64_t K, mgpuStream_t stream);
+/* output = act(input . weight + bias) + residual; replaces mgpuMatmulEx<T>
+ * (Ops.h:51-55; Ops.cu:134-234).  hasRelu: 0 none, 1 ReLU; hasRelu == 2 selects
+ * GELU (erf form), which the reference does not have.  fp32 accumulation. */
+void mgpuMatmulExF16(void *input, void *weight, void *bias, void *output, void *residual,
+                     int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
+                     int32_t hasResidual, mgpuStream_t stream);
+void mgpuMatmulExF32(float *input, float *weight, float *bias, float *output, float *residual,
+                     int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
+                     int32_t hasResidual, mgpuStream_t stream);
+
+/* ---- transformer layers ----------------------------------------------- */
+/* Pre-LN layer, fp32 in/out, fp16 compute; same signature as the reference
+ * (Ops.h:43-48; lib/Kernels/GPU/LLM.cu:26-159). */
+void mgpuLLMDecodingContextLayer(float *input, float *qkv, float *gemm_weight, float *gemm_bias,
+                                 float *ffn1_weight, float *ffn1_bias, float *ffn2_weight,
+                                 float *ffn2_bias, float *output, int64_t batch, int64_t seq_len,
+                                 int64_t d_model, int64_t feed_forward_dim, int64_t head_num,
+                                 bool norm_first, bool is_casual, bool is_relu,
+                                 mgpuStream_t stream);
+
+/* Post-LN BERT encoder layer on fp16 tensors; no counterpart in the reference
+ * (its only layer entry point is the pre-LN one above):
+ *   qkv = x . wqkv + bqkv                 [M, 3d] read as [B,S,3,H,64]
+ *   ctx = fused MHA(qkv, seqlens)         scale 1/8, no causal mask
+ *   h1  = LayerNorm(ctx . wo + bo + x)    gamma1, beta1
+ *   f   = GELU_erf(h1 . w1 + b1)
+ *   out = LayerNorm(f . w2 + b2 + h1)     gamma2, beta2
+ * Weights are row major [in, out]; seqlens may be NULL. */
+void mgpuBertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, const void *wo,
+                             const void *bo, const void *gamma1, const void *beta1, const void *w1,
+                             const void *b1, const void *w2, const void *b2, const void *gamma2,
+                             const void *beta2, const int32_t *seqlens, void *out, int64_t batch,
+                             int64_t seq_len, int64_t d_model, int64_t feed_forward_dim,
+                             int64_t head_num, float eps, mgpuStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MGPU_OPS_H_ */

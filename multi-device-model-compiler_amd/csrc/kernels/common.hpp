@@ -1,0 +1,75 @@
+// Shared helpers of the device kernel library: error convention, launch
+// geometry and cross-lane reductions for 64-wide wavefronts.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <stdexcept>
+#include <string>
+
+namespace mgpu {
+
+// Error convention of the kernel library: print, then throw std::logic_error
+// (reference: lib/Kernels/GPU/Ops.cu:21-41).  The extern "C" layer catches it.
+[[noreturn]] inline void fail(const std::string &what) {
+  std::fprintf(stderr, "mgpu ops: %s\n", what.c_str());
+  throw std::logic_error(what);
+}
+
+inline void checkHipStatus(hipError_t status, const char *where) {
+  if (status != hipSuccess) {
+    (void)hipGetLastError();
+    fail(std::string(where) + ": HIP API failed with status " +
+         std::to_string(static_cast<int>(status)) + ": " + hipGetErrorString(status));
+  }
+}
+
+#define MGPU_CHECK_HIP(expr) ::mgpu::checkHipStatus((expr), #expr)
+#define MGPU_CHECK_LAUNCH(name) ::mgpu::checkHipStatus(hipGetLastError(), name)
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int numComputeUnits() {
+  static int cus = [] {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    return v;
+  }();
+  return cus;
+}
+
+// ---- cross-lane sums on a 64-wide wavefront ------------------------------
+// DPP moves inside a row of 16 lanes (no LDS traffic), then lane exchanges
+// across rows.  After the call every participating lane holds the same sum.
+
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+
+// Sum over groups of LANES consecutive lanes (LANES in {16, 32, 64}).
+template <int LANES> __device__ __forceinline__ float group_sum(float v) {
+  v += dpp_move<0xB1>(v);  // quad_perm [1,0,3,2]: xor 1
+  v += dpp_move<0x4E>(v);  // quad_perm [2,3,0,1]: xor 2
+  v += dpp_move<0x141>(v); // row_half_mirror: lane i <-> 7 - i
+  v += dpp_move<0x140>(v); // row_mirror:      lane i <-> 15 - i
+  if (LANES >= 32) v += __shfl_xor(v, 16);
+  if (LANES >= 64) v += __shfl_xor(v, 32);
+  return v;
+}
+
+template <int LANES> __device__ __forceinline__ float group_max(float v) {
+  v = fmaxf(v, dpp_move<0xB1>(v));
+  v = fmaxf(v, dpp_move<0x4E>(v));
+  v = fmaxf(v, dpp_move<0x141>(v));
+  v = fmaxf(v, dpp_move<0x140>(v));
+  if (LANES >= 32) v = fmaxf(v, __shfl_xor(v, 16));
+  if (LANES >= 64) v = fmaxf(v, __shfl_xor(v, 32));
+  return v;
+}
+
+} // namespace mgpu

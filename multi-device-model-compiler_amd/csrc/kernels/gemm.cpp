@@ -1,0 +1,165 @@
+// GEMM with bias / activation / residual epilogue over hipBLASLt.
+//
+// Replaces mgpuMatmul and mgpuMatmulEx<T> (lib/Kernels/GPU/Ops.cu:57-120,
+// 134-234).  Same row-major contract through the column-major operand swap of
+// Ops.cu:83-85,178-183: out^T[N,M] = W^T[N,K] . in^T[K,M].  Differences:
+//  * the whole plan (operation descriptor, layouts, chosen algorithm) is built
+//    once per (shape, flags, type) and reused; the reference rebuilds all
+//    descriptors on every call and caches only the heuristic result;
+//  * fp16 / bf16 inputs accumulate in fp32 (HIPBLAS_COMPUTE_32F); the reference
+//    asks for fp16 accumulation (Ops.cu:164-167);
+//  * GELU is applied by an exact-erf kernel after a bias-only epilogue, because
+//    the library's fused GELU is the tanh approximation.
+#include "common.hpp"
+#include "mgpu_ops_internal.hpp"
+
+#include <hipblaslt/hipblaslt.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+
+namespace mgpu {
+
+namespace {
+
+hipblasLtHandle_t ltHandle = nullptr;
+void *workspace = nullptr;
+constexpr size_t workspaceSize = 32u * 1024u * 1024u;
+std::mutex planMutex;
+
+void checkBlas(hipblasStatus_t status, const char *where) {
+  if (status != HIPBLAS_STATUS_SUCCESS)
+    fail(std::string(where) + ": hipBLASLt API failed with status " + std::to_string((int)status));
+}
+#define MGPU_CHECK_BLAS(expr) checkBlas((expr), #expr)
+
+struct Plan {
+  hipblasLtMatmulDesc_t op = nullptr;
+  hipblasLtMatrixLayout_t a = nullptr, b = nullptr, d = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+};
+
+using Key = std::tuple<int64_t, int64_t, int64_t, int, int, int, int>;
+std::map<Key, Plan> plans;
+
+hipDataType dataType(DType dt) {
+  switch (dt) {
+  case DType::F32:
+    return HIP_R_32F;
+  case DType::F16:
+    return HIP_R_16F;
+  default:
+    return HIP_R_16BF;
+  }
+}
+
+void destroyPlan(Plan &p) {
+  if (p.d) hipblasLtMatrixLayoutDestroy(p.d);
+  if (p.b) hipblasLtMatrixLayoutDestroy(p.b);
+  if (p.a) hipblasLtMatrixLayoutDestroy(p.a);
+  if (p.op) hipblasLtMatmulDescDestroy(p.op);
+  p = Plan{};
+}
+
+const Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, bool relu,
+                    bool hasResidual) {
+  const Key key{M, N, K, (int)hasBias, (int)relu, (int)hasResidual, (int)dt};
+  auto it = plans.find(key);
+  if (it != plans.end()) return it->second;
+
+  Plan p;
+  const hipDataType t = dataType(dt);
+  MGPU_CHECK_BLAS(hipblasLtMatmulDescCreate(&p.op, HIPBLAS_COMPUTE_32F, HIP_R_32F));
+  hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_DEFAULT;
+  if (hasBias && relu)
+    epilogue = HIPBLASLT_EPILOGUE_RELU_BIAS;
+  else if (hasBias)
+    epilogue = HIPBLASLT_EPILOGUE_BIAS;
+  else if (relu)
+    epilogue = HIPBLASLT_EPILOGUE_RELU;
+  MGPU_CHECK_BLAS(hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue,
+                                                  sizeof(epilogue)));
+  if (hasBias) {
+    const int32_t biasType = (int32_t)t;
+    MGPU_CHECK_BLAS(hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE,
+                                                    &biasType, sizeof(biasType)));
+  }
+  // Column-major view of the row-major operands: A = weight (N x K, ld N),
+  // B = input (K x M, ld K), C/D = output (N x M, ld N).
+  MGPU_CHECK_BLAS(hipblasLtMatrixLayoutCreate(&p.a, t, N, K, N));
+  MGPU_CHECK_BLAS(hipblasLtMatrixLayoutCreate(&p.b, t, K, M, K));
+  MGPU_CHECK_BLAS(hipblasLtMatrixLayoutCreate(&p.d, t, N, M, N));
+
+  hipblasLtMatmulPreference_t pref = nullptr;
+  MGPU_CHECK_BLAS(hipblasLtMatmulPreferenceCreate(&pref));
+  const uint64_t ws = workspaceSize;
+  MGPU_CHECK_BLAS(hipblasLtMatmulPreferenceSetAttribute(
+      pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws)));
+  hipblasLtMatmulHeuristicResult_t result = {};
+  int returned = 0;
+  // A dummy non-null bias pointer lets the heuristic see the bias epilogue.
+  const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(ltHandle, p.op, p.a, p.b, p.d, p.d,
+                                                             pref, 1, &result, &returned);
+  hipblasLtMatmulPreferenceDestroy(pref);
+  if (st != HIPBLAS_STATUS_SUCCESS || returned == 0) {
+    destroyPlan(p);
+    fail("matmul: hipBLASLt has no algorithm for M=" + std::to_string(M) + " N=" +
+         std::to_string(N) + " K=" + std::to_string(K));
+  }
+  p.algo = result.algo;
+  return plans.emplace(key, p).first->second;
+}
+
+} // namespace
+
+void gemmInit() {
+  if (ltHandle) return;
+  MGPU_CHECK_BLAS(hipblasLtCreate(&ltHandle));
+  MGPU_CHECK_HIP(hipMalloc(&workspace, workspaceSize));
+}
+
+void gemmDeinit() {
+  std::lock_guard<std::mutex> lock(planMutex);
+  for (auto &kv : plans) destroyPlan(kv.second);
+  plans.clear();
+  if (workspace) (void)hipFree(workspace);
+  workspace = nullptr;
+  if (ltHandle) hipblasLtDestroy(ltHandle);
+  ltHandle = nullptr;
+}
+
+void matmulEx(DType dt, const void *input, const void *weight, const void *bias, void *output,
+              const void *residual, int64_t M, int64_t N, int64_t K, bool hasBias, int act,
+              bool hasResidual, hipStream_t stream) {
+  if (M < 0 || N < 0 || K < 0) fail("matmul: negative shape");
+  if (M == 0 || N == 0) return;
+  if (K == 0) fail("matmul: K must be positive");
+  if (!ltHandle) fail("matmul: gpuOpsInit() has not been called");
+  if (!input || !weight || !output) fail("matmul: null pointer");
+  if (hasBias && !bias) fail("matmul: hasBias set but bias is null");
+  if (hasResidual && !residual) fail("matmul: hasResidual set but residual is null");
+  if (act < ACT_NONE || act > ACT_GELU) fail("matmul: unknown activation");
+  if (act != ACT_NONE && hasResidual)
+    fail("matmul: an activation cannot be combined with a residual");
+
+  std::lock_guard<std::mutex> lock(planMutex);
+  const Plan &p = getPlan(dt, M, N, K, hasBias, act == ACT_RELU, hasResidual);
+  if (hasBias)
+    MGPU_CHECK_BLAS(hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias,
+                                                    sizeof(bias)));
+  const float alpha = 1.0f, beta = hasResidual ? 1.0f : 0.0f;
+  MGPU_CHECK_BLAS(hipblasLtMatmul(ltHandle, p.op, &alpha, weight, p.a, input, p.b, &beta,
+                                  hasResidual ? residual : output, p.d, output, p.d, &p.algo,
+                                  workspace, workspaceSize, stream));
+  if (act == ACT_GELU) {
+    if (dt == DType::F16)
+      geluInPlaceF16(output, (size_t)M * N, stream);
+    else if (dt == DType::F32)
+      geluInPlaceF32(static_cast<float *>(output), (size_t)M * N, stream);
+    else
+      fail("matmul: GELU epilogue is built for fp16 and fp32 only");
+  }
+}
+
+} // namespace mgpu

@@ -1,0 +1,267 @@
+// LayerNorm and add-residual + LayerNorm for fp32 / fp16 / bf16 rows.
+//
+// Replaces generalAddBiasResidualLayerNormOpt2 and its dispatch ladder
+// (lib/Kernels/GPU/LayerNorm.cu:138-260,262-466).  The reference keeps the row
+// in shared memory, writes the output twice and needs two block barriers; here
+// a row lives in the registers of one group of 16/32/64 lanes:
+//   one 128-bit coalesced load per vector, statistics in fp32 with a two-pass
+//   (mean, then centred sum of squares) reduction over registers and DPP /
+//   lane-exchange sums, one 128-bit store per vector.  One pass over HBM.
+// Rows wider than a wavefront can hold, rows whose length is not a multiple of
+// the vector width, and unaligned pointers take a block-per-row kernel.
+#include "common.hpp"
+#include "mgpu_ops_internal.hpp"
+#include "types.hpp"
+
+namespace mgpu {
+
+namespace {
+
+constexpr int kMaxVPL = 8; // vectors per lane the register kernel is built for
+
+// One group of LANES lanes owns one row: lane l holds vectors l, l+LANES, ...
+// (VPL of them, the last ones predicated off when the row is shorter).
+template <typename T, int LANES, int VPL, bool RESIDUAL>
+__global__ __launch_bounds__(256) void layernorm_rows_kernel(
+    const T *__restrict__ input, const T *__restrict__ residual, const T *__restrict__ gamma,
+    const T *__restrict__ beta, T *__restrict__ sumOut, T *__restrict__ normed, float eps, int m,
+    int n) {
+  using Tr = ElemTraits<T>;
+  constexpr int VEC = Tr::kVec; // elements per 16-byte vector
+  constexpr int GROUPS = 256 / LANES;
+  const int lane = threadIdx.x % LANES;
+  const int group = threadIdx.x / LANES;
+  const int nvec = n / VEC;
+  const float inv_n = 1.0f / (float)n;
+
+  const u32x4 *gv = reinterpret_cast<const u32x4 *>(gamma);
+  const u32x4 *bv = reinterpret_cast<const u32x4 *>(beta);
+
+  for (int row = blockIdx.x * GROUPS + group; row < m; row += gridDim.x * GROUPS) {
+    const u32x4 *xv = reinterpret_cast<const u32x4 *>(input + (size_t)row * n);
+    const u32x4 *rv = RESIDUAL ? reinterpret_cast<const u32x4 *>(residual + (size_t)row * n) : nullptr;
+
+    u32x4 raw[VPL], rawr[VPL];
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = lane + k * LANES;
+      if (v < nvec) {
+        raw[k] = __builtin_nontemporal_load(xv + v);
+        if (RESIDUAL) rawr[k] = __builtin_nontemporal_load(rv + v);
+      }
+    }
+
+    float x[VPL][VEC];
+    float sum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = lane + k * LANES;
+      if (v < nvec) {
+        Tr::unpack(raw[k], x[k]);
+        if (RESIDUAL) {
+          float r[VEC];
+          Tr::unpack(rawr[k], r);
+#pragma unroll
+          for (int e = 0; e < VEC; e++) x[k][e] += r[e];
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; e++) sum += x[k][e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) x[k][e] = 0.0f;
+      }
+    }
+    const float mean = group_sum<LANES>(sum) * inv_n;
+
+    float sq = 0.0f;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = lane + k * LANES;
+      if (v < nvec) {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+          const float d = x[k][e] - mean;
+          sq += d * d;
+        }
+      }
+    }
+    const float var = group_sum<LANES>(sq) * inv_n;
+    const float rstd = 1.0f / sqrtf(var + eps);
+
+    u32x4 *yv = reinterpret_cast<u32x4 *>(normed + (size_t)row * n);
+    u32x4 *sv = RESIDUAL ? reinterpret_cast<u32x4 *>(sumOut + (size_t)row * n) : nullptr;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = lane + k * LANES;
+      if (v < nvec) {
+        float g[VEC], b[VEC], y[VEC];
+        Tr::unpack(gv[v], g);
+        Tr::unpack(bv[v], b);
+        if (RESIDUAL) {
+          // The sum is stored rounded to T and the normalised value is taken
+          // from that rounded sum, while mean and variance came from the
+          // un-rounded fp32 sums (reference dataflow, LayerNorm.cu:203-233).
+          const u32x4 packed = Tr::pack(x[k]);
+          __builtin_nontemporal_store(packed, sv + v);
+          Tr::unpack(packed, x[k]);
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; e++) y[e] = (x[k][e] - mean) * rstd * g[e] + b[e];
+        __builtin_nontemporal_store(Tr::pack(y), yv + v);
+      }
+    }
+  }
+}
+
+// Any n, any alignment: one 256-thread block per row, three sweeps over the
+// row (the second and third hit in cache).
+template <typename T, bool RESIDUAL>
+__global__ __launch_bounds__(256) void layernorm_general_kernel(
+    const T *__restrict__ input, const T *__restrict__ residual, const T *__restrict__ gamma,
+    const T *__restrict__ beta, T *__restrict__ sumOut, T *__restrict__ normed, float eps, int m,
+    int n) {
+  using Tr = ElemTraits<T>;
+  __shared__ float partial[4];
+  const int wave = threadIdx.x / 64;
+  const float inv_n = 1.0f / (float)n;
+  for (int row = blockIdx.x; row < m; row += gridDim.x) {
+    const T *xr = input + (size_t)row * n;
+    const T *rr = RESIDUAL ? residual + (size_t)row * n : nullptr;
+    auto value = [&](int i) {
+      float v = Tr::toFloat(xr[i]);
+      if (RESIDUAL) v += Tr::toFloat(rr[i]);
+      return v;
+    };
+    float sum = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 256) sum += value(i);
+    sum = group_sum<64>(sum);
+    __syncthreads();
+    if (threadIdx.x % 64 == 0) partial[wave] = sum;
+    __syncthreads();
+    const float mean = (partial[0] + partial[1] + partial[2] + partial[3]) * inv_n;
+    float sq = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 256) {
+      const float d = value(i) - mean;
+      sq += d * d;
+    }
+    sq = group_sum<64>(sq);
+    __syncthreads();
+    if (threadIdx.x % 64 == 0) partial[wave] = sq;
+    __syncthreads();
+    const float var = (partial[0] + partial[1] + partial[2] + partial[3]) * inv_n;
+    const float rstd = 1.0f / sqrtf(var + eps);
+    for (int i = threadIdx.x; i < n; i += 256) {
+      float v = value(i);
+      if (RESIDUAL) {
+        const T rounded = Tr::fromFloat(v);
+        sumOut[(size_t)row * n + i] = rounded;
+        v = Tr::toFloat(rounded);
+      }
+      normed[(size_t)row * n + i] =
+          Tr::fromFloat((v - mean) * rstd * Tr::toFloat(gamma[i]) + Tr::toFloat(beta[i]));
+    }
+  }
+}
+
+template <typename T, int LANES, int VPL, bool RESIDUAL>
+void launchRows(const T *input, const T *residual, const T *gamma, const T *beta, T *sumOut,
+                T *normed, float eps, int m, int n, hipStream_t stream) {
+  constexpr int GROUPS = 256 / LANES;
+  int64_t blocks = ((int64_t)m + GROUPS - 1) / GROUPS;
+  const int64_t cap = (int64_t)numComputeUnits() * 8;
+  if (blocks > cap) blocks = cap;
+  layernorm_rows_kernel<T, LANES, VPL, RESIDUAL><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+      input, residual, gamma, beta, sumOut, normed, eps, m, n);
+  MGPU_CHECK_LAUNCH("layernorm_rows_kernel");
+}
+
+template <typename T, int LANES, bool RESIDUAL>
+void dispatchVPL(int vpl, const T *input, const T *residual, const T *gamma, const T *beta,
+                 T *sumOut, T *normed, float eps, int m, int n, hipStream_t stream) {
+  switch (vpl) {
+#define MGPU_LN_CASE(V)                                                                          \
+  case V:                                                                                        \
+    launchRows<T, LANES, V, RESIDUAL>(input, residual, gamma, beta, sumOut, normed, eps, m, n,   \
+                                      stream);                                                   \
+    break;
+    MGPU_LN_CASE(1)
+    MGPU_LN_CASE(2)
+    MGPU_LN_CASE(3)
+    MGPU_LN_CASE(4)
+    MGPU_LN_CASE(5)
+    MGPU_LN_CASE(6)
+    MGPU_LN_CASE(7)
+    MGPU_LN_CASE(8)
+#undef MGPU_LN_CASE
+  default:
+    fail("layerNorm: internal dispatch error");
+  }
+}
+
+template <typename T, bool RESIDUAL>
+void layerNormTyped(const T *input, const T *residual, const T *gamma, const T *beta, T *sumOut,
+                    T *normed, float eps, int m, int n, hipStream_t stream) {
+  constexpr int VEC = ElemTraits<T>::kVec;
+  const bool vectorOk = n % VEC == 0 && aligned16(input) && aligned16(gamma) && aligned16(beta) &&
+                        aligned16(normed) && (!RESIDUAL || (aligned16(residual) && aligned16(sumOut)));
+  const int nvec = n / VEC;
+  if (vectorOk && nvec <= 64 * kMaxVPL) {
+    // Smallest lane group that keeps at most 4 vectors per lane; wider rows
+    // use the whole wavefront with up to kMaxVPL vectors per lane.
+    if (nvec <= 16 * 4)
+      dispatchVPL<T, 16, RESIDUAL>((nvec + 15) / 16, input, residual, gamma, beta, sumOut, normed,
+                                   eps, m, n, stream);
+    else if (nvec <= 32 * 4)
+      dispatchVPL<T, 32, RESIDUAL>((nvec + 31) / 32, input, residual, gamma, beta, sumOut, normed,
+                                   eps, m, n, stream);
+    else
+      dispatchVPL<T, 64, RESIDUAL>((nvec + 63) / 64, input, residual, gamma, beta, sumOut, normed,
+                                   eps, m, n, stream);
+    return;
+  }
+  int64_t blocks = m;
+  const int64_t cap = (int64_t)numComputeUnits() * 8;
+  if (blocks > cap) blocks = cap;
+  layernorm_general_kernel<T, RESIDUAL><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+      input, residual, gamma, beta, sumOut, normed, eps, m, n);
+  MGPU_CHECK_LAUNCH("layernorm_general_kernel");
+}
+
+template <typename T>
+void layerNormDispatch(const void *input, const void *residual, const void *gamma,
+                       const void *beta, void *sumOut, void *normed, float eps, int m, int n,
+                       hipStream_t stream) {
+  if (residual)
+    layerNormTyped<T, true>(static_cast<const T *>(input), static_cast<const T *>(residual),
+                            static_cast<const T *>(gamma), static_cast<const T *>(beta),
+                            static_cast<T *>(sumOut), static_cast<T *>(normed), eps, m, n, stream);
+  else
+    layerNormTyped<T, false>(static_cast<const T *>(input), nullptr, static_cast<const T *>(gamma),
+                             static_cast<const T *>(beta), nullptr, static_cast<T *>(normed), eps,
+                             m, n, stream);
+}
+
+} // namespace
+
+void layerNorm(DType dt, const void *input, const void *residual, const void *gamma,
+               const void *beta, void *sumOut, void *normed, float eps, int m, int n,
+               hipStream_t stream) {
+  if (m < 0 || n < 0) fail("layerNorm: negative shape");
+  if (m == 0 || n == 0) return;
+  if (!input || !gamma || !beta || !normed) fail("layerNorm: null pointer");
+  if ((residual == nullptr) != (sumOut == nullptr))
+    fail("layerNorm: residual and sum output must be given together");
+  switch (dt) {
+  case DType::F32:
+    layerNormDispatch<float>(input, residual, gamma, beta, sumOut, normed, eps, m, n, stream);
+    break;
+  case DType::F16:
+    layerNormDispatch<_Float16>(input, residual, gamma, beta, sumOut, normed, eps, m, n, stream);
+    break;
+  case DType::BF16:
+    layerNormDispatch<bf16_t>(input, residual, gamma, beta, sumOut, normed, eps, m, n, stream);
+    break;
+  }
+}
+
+} // namespace mgpu

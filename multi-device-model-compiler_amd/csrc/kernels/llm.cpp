@@ -1,0 +1,189 @@
+// Transformer layers composed from the kernels of this library.
+//
+// decodingContextLayer is the counterpart of mgpuLLMDecodingContextLayer
+// (lib/Kernels/GPU/LLM.cu:26-159): fp32 tensors in and out, fp16 compute,
+// weight casts on a side stream overlapped with compute through one event.
+// Kept from the reference: the dataflow (pre-LN, gamma = 1 / beta = 0
+// LayerNorms at eps 1e-5, packed-QKV attention, bias epilogues, residual
+// through the GEMM's C operand).  Changed on purpose:
+//  * head_num, is_casual and is_relu are honoured (the reference ignores them
+//    and runs 8 heads x 128, causal, ReLU: LLM.cu:18-19,79-81,119-121);
+//  * one stream-ordered arena instead of 12 allocations and frees per call;
+//  * the side stream first waits for work already queued on the caller's
+//    stream, and the final fp16 -> fp32 cast runs after the last GEMM on the
+//    caller's stream (the reference issues it on the side stream without
+//    waiting for that GEMM: LLM.cu:136-141).
+//
+// bertEncoderLayerF16 is the post-LN BERT encoder layer on fp16 tensors (GELU,
+// learned LayerNorm affine, optional key-padding lengths); the reference has
+// no such entry point.
+#include "common.hpp"
+#include "mgpu_ops_internal.hpp"
+
+namespace mgpu {
+
+namespace {
+
+hipStream_t copyStream = nullptr;
+hipEvent_t copyEvent = nullptr;
+hipEvent_t forkEvent = nullptr;
+
+// Bump allocator over one stream-ordered allocation; every slice is 256-byte
+// aligned so all vectorised kernels see aligned pointers.
+class Arena {
+public:
+  size_t reserve(size_t bytes) {
+    const size_t at = total_;
+    total_ += (bytes + 255) & ~size_t(255);
+    return at;
+  }
+  void allocate(hipStream_t s) { MGPU_CHECK_HIP(hipMallocAsync(&base_, total_ ? total_ : 256, s)); }
+  void release(hipStream_t s) {
+    if (base_) MGPU_CHECK_HIP(hipFreeAsync(base_, s));
+    base_ = nullptr;
+  }
+  template <typename T = void> T *at(size_t offset) const {
+    return reinterpret_cast<T *>(static_cast<char *>(base_) + offset);
+  }
+
+private:
+  void *base_ = nullptr;
+  size_t total_ = 0;
+};
+
+} // namespace
+
+void llmInit() {
+  if (copyStream) return;
+  MGPU_CHECK_HIP(hipStreamCreateWithFlags(&copyStream, hipStreamNonBlocking));
+  MGPU_CHECK_HIP(hipEventCreateWithFlags(&copyEvent, hipEventDisableTiming));
+  MGPU_CHECK_HIP(hipEventCreateWithFlags(&forkEvent, hipEventDisableTiming));
+}
+
+void llmDeinit() {
+  if (copyStream) (void)hipStreamDestroy(copyStream);
+  if (copyEvent) (void)hipEventDestroy(copyEvent);
+  if (forkEvent) (void)hipEventDestroy(forkEvent);
+  copyStream = nullptr;
+  copyEvent = forkEvent = nullptr;
+}
+
+void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *gemm_bias,
+                          float *ffn1_weight, float *ffn1_bias, float *ffn2_weight,
+                          float *ffn2_bias, float *output, int64_t batch, int64_t seq_len,
+                          int64_t d_model, int64_t ffn, int64_t heads, bool /*norm_first*/,
+                          bool causal, bool relu, hipStream_t stream) {
+  if (!copyStream) fail("mgpuLLMDecodingContextLayer: gpuOpsInit() has not been called");
+  if (batch < 0 || seq_len < 0 || d_model <= 0 || ffn <= 0 || heads <= 0)
+    fail("mgpuLLMDecodingContextLayer: bad shape");
+  if (d_model % heads || d_model / heads != 64)
+    fail("mgpuLLMDecodingContextLayer: d_model / head_num must be 64");
+  if (batch == 0 || seq_len == 0) return;
+  if (!input || !qkv || !gemm_weight || !gemm_bias || !ffn1_weight || !ffn1_bias || !ffn2_weight ||
+      !ffn2_bias || !output)
+    fail("mgpuLLMDecodingContextLayer: null pointer");
+  const int64_t M = batch * seq_len, d = d_model;
+  if (M > 0x7fffffff || d > 0x7fffffff) fail("mgpuLLMDecodingContextLayer: shape too large");
+  constexpr size_t h = 2; // bytes per fp16
+
+  Arena arena;
+  const size_t oX = arena.reserve(M * d * h), oLn = arena.reserve(M * d * h);
+  const size_t oGamma = arena.reserve(d * h), oBeta = arena.reserve(d * h);
+  const size_t oWqkv = arena.reserve(d * 3 * d * h), oQkv = arena.reserve(M * 3 * d * h);
+  const size_t oWo = arena.reserve(d * d * h), oBo = arena.reserve(d * h);
+  const size_t oProj = arena.reserve(M * d * h), oY = arena.reserve(M * d * h);
+  const size_t oW1 = arena.reserve(d * ffn * h), oB1 = arena.reserve(ffn * h);
+  const size_t oF = arena.reserve(M * ffn * h);
+  const size_t oW2 = arena.reserve(ffn * d * h), oB2 = arena.reserve(d * h);
+  const size_t oOut = arena.reserve(M * d * h);
+
+  // Fork: the side stream may not run ahead of what already sits on `stream`.
+  MGPU_CHECK_HIP(hipEventRecord(forkEvent, stream));
+  MGPU_CHECK_HIP(hipStreamWaitEvent(copyStream, forkEvent, 0));
+  arena.allocate(copyStream);
+  auto sync = [&] {
+    MGPU_CHECK_HIP(hipEventRecord(copyEvent, copyStream));
+    MGPU_CHECK_HIP(hipStreamWaitEvent(stream, copyEvent, 0));
+  };
+
+  castF32ToF16(arena.at(oX), input, M * d, copyStream);
+  fillF16(arena.at(oGamma), d, 1.0f, copyStream);
+  fillF16(arena.at(oBeta), d, 0.0f, copyStream);
+  sync();
+  layerNorm(DType::F16, arena.at(oX), nullptr, arena.at(oGamma), arena.at(oBeta), nullptr,
+            arena.at(oLn), 1e-5f, (int)M, (int)d, stream);
+
+  castF32ToF16(arena.at(oWqkv), qkv, d * 3 * d, copyStream);
+  sync();
+  matmulEx(DType::F16, arena.at(oLn), arena.at(oWqkv), nullptr, arena.at(oQkv), nullptr, M, 3 * d,
+           d, false, ACT_NONE, false, stream);
+
+  // Attention context overwrites the first LayerNorm output, like the reference.
+  fusedMHA(DType::F16, arena.at(oQkv), nullptr, arena.at(oLn), (int)batch, (int)seq_len,
+           (int)heads, 64, 0.125f, causal, stream);
+
+  castF32ToF16(arena.at(oWo), gemm_weight, d * d, copyStream);
+  castF32ToF16(arena.at(oBo), gemm_bias, d, copyStream);
+  sync();
+  matmulEx(DType::F16, arena.at(oLn), arena.at(oWo), arena.at(oBo), arena.at(oProj), nullptr, M, d,
+           d, true, ACT_NONE, false, stream);
+
+  layerNorm(DType::F16, arena.at(oProj), arena.at(oX), arena.at(oGamma), arena.at(oBeta),
+            arena.at(oY), arena.at(oLn), 1e-5f, (int)M, (int)d, stream);
+
+  castF32ToF16(arena.at(oW1), ffn1_weight, d * ffn, copyStream);
+  castF32ToF16(arena.at(oB1), ffn1_bias, ffn, copyStream);
+  sync();
+  matmulEx(DType::F16, arena.at(oLn), arena.at(oW1), arena.at(oB1), arena.at(oF), nullptr, M, ffn,
+           d, true, relu ? ACT_RELU : ACT_GELU, false, stream);
+
+  castF32ToF16(arena.at(oW2), ffn2_weight, ffn * d, copyStream);
+  castF32ToF16(arena.at(oB2), ffn2_bias, d, copyStream);
+  sync();
+  matmulEx(DType::F16, arena.at(oF), arena.at(oW2), arena.at(oB2), arena.at(oOut), arena.at(oY), M,
+           d, ffn, true, ACT_NONE, true, stream);
+
+  castF16ToF32(output, arena.at(oOut), M * d, stream);
+  arena.release(stream);
+}
+
+void bertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, const void *wo,
+                         const void *bo, const void *gamma1, const void *beta1, const void *w1,
+                         const void *b1, const void *w2, const void *b2, const void *gamma2,
+                         const void *beta2, const int32_t *seqlens, void *out, int64_t B,
+                         int64_t S, int64_t d, int64_t ffn, int64_t H, float eps,
+                         hipStream_t stream) {
+  if (B < 0 || S < 0 || d <= 0 || ffn <= 0 || H <= 0) fail("mgpuBertEncoderLayerF16: bad shape");
+  if (d % H || d / H != 64) fail("mgpuBertEncoderLayerF16: d_model / head_num must be 64");
+  if (B == 0 || S == 0) return;
+  if (!x || !wqkv || !bqkv || !wo || !bo || !gamma1 || !beta1 || !w1 || !b1 || !w2 || !b2 ||
+      !gamma2 || !beta2 || !out)
+    fail("mgpuBertEncoderLayerF16: null pointer");
+  const int64_t M = B * S;
+  if (M > 0x7fffffff) fail("mgpuBertEncoderLayerF16: shape too large");
+  constexpr size_t h = 2;
+
+  Arena arena;
+  const size_t oQkv = arena.reserve(M * 3 * d * h), oCtx = arena.reserve(M * d * h);
+  const size_t oProj = arena.reserve(M * d * h), oSum = arena.reserve(M * d * h);
+  const size_t oH1 = arena.reserve(M * d * h), oF = arena.reserve(M * ffn * h);
+  arena.allocate(stream);
+
+  matmulEx(DType::F16, x, wqkv, bqkv, arena.at(oQkv), nullptr, M, 3 * d, d, true, ACT_NONE, false,
+           stream);
+  fusedMHA(DType::F16, arena.at(oQkv), seqlens, arena.at(oCtx), (int)B, (int)S, (int)H, 64, 0.125f,
+           false, stream);
+  matmulEx(DType::F16, arena.at(oCtx), wo, bo, arena.at(oProj), nullptr, M, d, d, true, ACT_NONE,
+           false, stream);
+  layerNorm(DType::F16, arena.at(oProj), x, gamma1, beta1, arena.at(oSum), arena.at(oH1), eps,
+            (int)M, (int)d, stream);
+  matmulEx(DType::F16, arena.at(oH1), w1, b1, arena.at(oF), nullptr, M, ffn, d, true, ACT_GELU,
+           false, stream);
+  matmulEx(DType::F16, arena.at(oF), w2, b2, arena.at(oProj), nullptr, M, d, ffn, true, ACT_NONE,
+           false, stream);
+  layerNorm(DType::F16, arena.at(oProj), arena.at(oH1), gamma2, beta2, arena.at(oSum), out, eps,
+            (int)M, (int)d, stream);
+  arena.release(stream);
+}
+
+} // namespace mgpu

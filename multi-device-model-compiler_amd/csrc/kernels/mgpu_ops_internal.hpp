@@ -1,0 +1,58 @@
+// C++ entry points behind the extern "C" layer (c_api.cpp) and the template
+// wrappers of Kernels/GPU/Ops.h.  All of them enqueue on `stream` and throw
+// std::logic_error (after printing) on bad arguments or a failed launch.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace mgpu {
+
+enum class DType { F32 = 0, F16 = 1, BF16 = 2 };
+
+void addF32(const float *a, const float *b, float *c, int64_t n, hipStream_t stream);
+
+// residual / sumOut may be null (plain LayerNorm).
+void layerNorm(DType dt, const void *input, const void *residual, const void *gamma,
+               const void *beta, void *sumOut, void *normed, float eps, int m, int n,
+               hipStream_t stream);
+
+void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int B, int S, int H,
+              int D, float scale, bool causal, hipStream_t stream);
+
+void castF32ToF16(void *dst, const float *src, size_t size, hipStream_t stream);
+void castF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream);
+void fillF16(void *dst, size_t count, float value, hipStream_t stream);
+void fillI32(int32_t *dst, size_t count, int32_t value, hipStream_t stream);
+
+void addFusedQKVBiasTransposeF16(void *q, void *k, void *v, void *qkv, const void *bias, int B,
+                                 int S, int tokens, int H, int D, hipStream_t stream);
+
+enum Activation { ACT_NONE = 0, ACT_RELU = 1, ACT_GELU = 2 };
+void gemmInit();
+void gemmDeinit();
+void matmulEx(DType dt, const void *input, const void *weight, const void *bias, void *output,
+              const void *residual, int64_t M, int64_t N, int64_t K, bool hasBias, int act,
+              bool hasResidual, hipStream_t stream);
+
+void llmInit();
+void llmDeinit();
+void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *gemm_bias,
+                          float *ffn1_weight, float *ffn1_bias, float *ffn2_weight,
+                          float *ffn2_bias, float *output, int64_t batch, int64_t seq_len,
+                          int64_t d_model, int64_t ffn, int64_t heads, bool norm_first,
+                          bool causal, bool relu, hipStream_t stream);
+
+void bertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, const void *wo,
+                         const void *bo, const void *gamma1, const void *beta1, const void *w1,
+                         const void *b1, const void *w2, const void *b2, const void *gamma2,
+                         const void *beta2, const int32_t *seqlens, void *out, int64_t B,
+                         int64_t S, int64_t d, int64_t ffn, int64_t H, float eps,
+                         hipStream_t stream);
+
+void geluInPlaceF16(void *data, size_t n, hipStream_t stream);
+void geluInPlaceF32(float *data, size_t n, hipStream_t stream);
+
+} // namespace mgpu

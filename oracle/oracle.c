@@ -1,0 +1,529 @@
+/*
+ * CPU oracle for the device kernel library: TEST INFRASTRUCTURE ONLY.
+ *
+ * This file restates, in plain C, what the reference computes on the path
+ *   add -> LayerNorm -> fused multi-head attention -> encoder layer.
+ * It is the checker that the HIP kernels are compared with and the CPU
+ * baseline that bench.py times; the product library never links or calls it.
+ *
+ * Arithmetic policy: every function reads the same bytes the GPU reads
+ * (fp32, or fp16/bf16 bit patterns as uint16_t), evaluates the closed form in
+ * fp64 (or fp32 with fp64 accumulators) and returns fp32, so the checker is
+ * strictly more accurate than either the reference's fp16 kernels or ours.
+ *
+ * Pinning status of each function is listed next to it ("pinned by ...");
+ * the pins live in tests/test_oracle_*.py.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORACLE_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------ */
+/* 16-bit float helpers (bit exact, no hardware dependence)            */
+/* ------------------------------------------------------------------ */
+
+static inline float half_bits_to_float(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1fu;
+  uint32_t man = h & 0x3ffu;
+  uint32_t bits;
+  if (exp == 0) {
+    if (man == 0) {
+      bits = sign;
+    } else { /* subnormal: normalise */
+      int e = -1;
+      do {
+        man <<= 1;
+        e++;
+      } while (!(man & 0x400u));
+      man &= 0x3ffu;
+      bits = sign | ((uint32_t)(127 - 15 - e) << 23) | (man << 13);
+    }
+  } else if (exp == 31) {
+    bits = sign | 0x7f800000u | (man << 13);
+  } else {
+    bits = sign | ((exp + 112u) << 23) | (man << 13);
+  }
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+
+/* double -> binary16, round to nearest even, done directly from the double so
+ * that no intermediate fp32 rounding can double-round. */
+static inline uint16_t double_to_half_bits(double d) {
+  uint64_t b;
+  memcpy(&b, &d, 8);
+  uint16_t sign = (uint16_t)((b >> 48) & 0x8000u);
+  int64_t exp = (int64_t)((b >> 52) & 0x7ff);
+  uint64_t man = b & 0xfffffffffffffull;
+  if (exp == 0x7ff) { /* inf / nan */
+    return (uint16_t)(sign | 0x7c00u | (man ? 0x200u : 0));
+  }
+  if (exp == 0) return sign; /* double subnormal or zero -> signed zero */
+  int64_t e = exp - 1023; /* unbiased */
+  man |= 1ull << 52;      /* implicit one: value = man * 2^(e-52) */
+  if (e > 15) return (uint16_t)(sign | 0x7c00u);
+  int shift; /* how many low bits of the 53-bit significand are dropped */
+  if (e >= -14) {
+    shift = 42; /* keep 11 bits (1 + 10) */
+  } else {
+    shift = 42 + (int)(-14 - e); /* subnormal half */
+    if (shift > 54) return sign;
+  }
+  uint64_t kept = man >> shift;
+  uint64_t rem = man & ((1ull << shift) - 1);
+  uint64_t halfway = 1ull << (shift - 1);
+  if (rem > halfway || (rem == halfway && (kept & 1))) kept++;
+  uint32_t out;
+  if (e >= -14) {
+    /* kept in [1024, 2048]; the carry case bumps the exponent naturally */
+    out = (uint32_t)((e + 15) << 10) + (uint32_t)(kept - 1024);
+    if (out >= 0x7c00u) out = 0x7c00u;
+  } else {
+    out = (uint32_t)kept; /* subnormal (or rounds up to the smallest normal) */
+  }
+  return (uint16_t)(sign | out);
+}
+
+static inline float bf16_bits_to_float(uint16_t h) {
+  uint32_t bits = (uint32_t)h << 16;
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+
+static inline uint16_t float_to_bf16_bits(float f) {
+  uint32_t b;
+  memcpy(&b, &f, 4);
+  if ((b & 0x7f800000u) == 0x7f800000u && (b & 0x7fffffu))
+    return (uint16_t)((b >> 16) | 0x40u);
+  uint32_t lsb = (b >> 16) & 1u;
+  b += 0x7fffu + lsb;
+  return (uint16_t)(b >> 16);
+}
+
+/* kind: 0 = fp32, 1 = fp16 bits, 2 = bf16 bits */
+static inline double load_elem(const void *p, int64_t i, int kind) {
+  switch (kind) {
+  case 0:
+    return (double)((const float *)p)[i];
+  case 1:
+    return (double)half_bits_to_float(((const uint16_t *)p)[i]);
+  default:
+    return (double)bf16_bits_to_float(((const uint16_t *)p)[i]);
+  }
+}
+
+static inline double round_to_kind(double v, int kind) {
+  switch (kind) {
+  case 0:
+    return (double)(float)v;
+  case 1:
+    return (double)half_bits_to_float(double_to_half_bits(v));
+  default:
+    return (double)bf16_bits_to_float(float_to_bf16_bits((float)v));
+  }
+}
+
+ORACLE_API void oracle_half_to_float(const uint16_t *src, float *dst, int64_t n) {
+  for (int64_t i = 0; i < n; i++) dst[i] = half_bits_to_float(src[i]);
+}
+
+/* pinned by: exhaustive comparison with numpy.float16 over all 65536 patterns
+ * and over random doubles incl. halfway cases. */
+ORACLE_API void oracle_double_to_half(const double *src, uint16_t *dst, int64_t n) {
+  for (int64_t i = 0; i < n; i++) dst[i] = double_to_half_bits(src[i]);
+}
+
+ORACLE_API void oracle_bf16_to_float(const uint16_t *src, float *dst, int64_t n) {
+  for (int64_t i = 0; i < n; i++) dst[i] = bf16_bits_to_float(src[i]);
+}
+
+ORACLE_API void oracle_float_to_bf16(const float *src, uint16_t *dst, int64_t n) {
+  for (int64_t i = 0; i < n; i++) dst[i] = float_to_bf16_bits(src[i]);
+}
+
+ORACLE_API int oracle_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+ORACLE_API void oracle_set_num_threads(int n) {
+#ifdef _OPENMP
+  omp_set_num_threads(n);
+#else
+  (void)n;
+#endif
+}
+
+/* ------------------------------------------------------------------ */
+/* Elementwise add                                                     */
+/* ------------------------------------------------------------------ */
+
+/* C = A + B in IEEE binary32, round to nearest even, one rounding per element.
+ * Follows examples/add.ll:42-66 (a 3 x 640 x 40 nest of 16-wide fadd, which is
+ * elementwise and order free).  Single threaded like that artefact.
+ * pinned by: oracle/_ref (add.ll compiled with llc), the committed golden
+ * sample drawn from it, numpy.add, and IEEE special values. */
+ORACLE_API void oracle_add_f32(const float *a, const float *b, float *c, int64_t n) {
+  for (int64_t i = 0; i < n; i++) c[i] = a[i] + b[i];
+}
+
+/* The same loop split over OpenMP threads; only used as a multi-core CPU
+ * baseline in the bench, never as the checker. */
+ORACLE_API void oracle_add_f32_mt(const float *a, const float *b, float *c, int64_t n) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; i++) c[i] = a[i] + b[i];
+}
+
+/* ------------------------------------------------------------------ */
+/* LayerNorm                                                           */
+/* ------------------------------------------------------------------ */
+
+/* y[r, :] = (x[r, :] - mean) / sqrt(var + eps) * gamma + beta over the last
+ * dim, biased variance.  Semantics of lib/Kernels/GPU/LayerNorm.cu:138-260
+ * (mean = sum/n at :217, rsqrt(E[x^2] - mean^2 + eps) at :218, affine at
+ * :230-233) with eps = 1e-5 at the call sites lib/Kernels/GPU/LLM.cu:50-52.
+ * Evaluated in fp64 with a two-pass variance; the result is returned in fp32.
+ * gamma / beta may be NULL (treated as 1 / 0), which is the use_affine=false
+ * LayerNorm of lib/Kernels/CPU/LLM.cpp:222-225.
+ * kind: 0 = fp32, 1 = fp16 bits, 2 = bf16 bits for x, gamma, beta.
+ * pinned by: torch.nn.functional.layer_norm (fp64 on CPU), hand-computed
+ * rows of n = 2, 4, 6, constant-row and shift-invariance identities. */
+ORACLE_API void oracle_layernorm(const void *x, const void *gamma, const void *beta, float *y,
+                                 double eps, int64_t m, int64_t n, int kind) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < m; r++) {
+    double sum = 0.0;
+    for (int64_t i = 0; i < n; i++) sum += load_elem(x, r * n + i, kind);
+    double mean = sum / (double)n;
+    double sq = 0.0;
+    for (int64_t i = 0; i < n; i++) {
+      double d = load_elem(x, r * n + i, kind) - mean;
+      sq += d * d;
+    }
+    double rstd = 1.0 / sqrt(sq / (double)n + eps);
+    for (int64_t i = 0; i < n; i++) {
+      double g = gamma ? load_elem(gamma, i, kind) : 1.0;
+      double b = beta ? load_elem(beta, i, kind) : 0.0;
+      y[r * n + i] = (float)((load_elem(x, r * n + i, kind) - mean) * rstd * g + b);
+    }
+  }
+}
+
+/* sum = round_kind(fp32(input) + fp32(residual)); normed = LN(sum) where the
+ * statistics come from the UN-rounded fp32 sums and the normalised value from
+ * the rounded one, exactly the dataflow of lib/Kernels/GPU/LayerNorm.cu:186-233
+ * (val_1 accumulates in float :172-201, tmp = cast(val) stored to shmem and
+ * output :203-207, x_sum / x2_sum use val :208-209, normalise reads shmem
+ * :230).  out_sum receives the rounded sums as fp32 values.
+ * pinned by: reduces to oracle_layernorm when residual == 0; the sum output is
+ * the closed form fp16(fp32(a)+fp32(b)) checked against numpy. */
+ORACLE_API void oracle_add_residual_layernorm(const void *input, const void *residual,
+                                              const void *gamma, const void *beta,
+                                              float *out_sum, float *normed, double eps,
+                                              int64_t m, int64_t n, int kind) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < m; r++) {
+    double sum = 0.0;
+    for (int64_t i = 0; i < n; i++) {
+      float s = (float)load_elem(input, r * n + i, kind) + (float)load_elem(residual, r * n + i, kind);
+      sum += (double)s;
+    }
+    double mean = sum / (double)n;
+    double sq = 0.0;
+    for (int64_t i = 0; i < n; i++) {
+      float s = (float)load_elem(input, r * n + i, kind) + (float)load_elem(residual, r * n + i, kind);
+      double d = (double)s - mean;
+      sq += d * d;
+    }
+    double rstd = 1.0 / sqrt(sq / (double)n + eps);
+    for (int64_t i = 0; i < n; i++) {
+      float s = (float)load_elem(input, r * n + i, kind) + (float)load_elem(residual, r * n + i, kind);
+      double sr = round_to_kind((double)s, kind);
+      out_sum[r * n + i] = (float)sr;
+      double g = gamma ? load_elem(gamma, i, kind) : 1.0;
+      double b = beta ? load_elem(beta, i, kind) : 0.0;
+      normed[r * n + i] = (float)((sr - mean) * rstd * g + b);
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ */
+/* Fused multi-head attention                                          */
+/* ------------------------------------------------------------------ */
+
+/* O[b, i, h, :] = sum_j softmax_j(scale * <Q[b,i,h,:], K[b,j,h,:]> + mask) V[b,j,h,:]
+ *
+ * qkv is packed [B, S, 3, H, D] (the reshape of lib/Kernels/CPU/LLM.cpp:243-246;
+ * per-token row of 3*H*D elements as in
+ * 3rdparty/trt_fused_multihead_attention/qkvToContext.cu:153,181), out is
+ * [B, S, H*D] (qkvToContext.cu:155,182; LLM.cpp transpose {0,2,1,3} + reshape).
+ * scale is the softmax scale 1/sqrt(D) of qkvToContext.cu:36-42,164-171.
+ * seqlens (may be NULL) holds B valid key counts: keys j >= seqlens[b] are
+ * excluded, every one of the S query rows is still computed (additive key
+ * mask of lib/Conversion/ConvertONNXToDevice/MultiHeadAttentionLayer.cpp:43-55).
+ * causal != 0 additionally excludes j > i (the flag of LLM.cu:79-81).
+ * A row with no admissible key yields zeros.
+ * Inputs are widened to fp32, dot products and softmax sums run in fp64.
+ * kind: 1 = fp16 bits, 2 = bf16 bits, 0 = fp32.
+ * pinned by: torch scaled_dot_product_attention (CPU fp64), brute-force python
+ * loops on S <= 8, rows-sum-to-one / constant-V / zero-Q / key-permutation
+ * identities.  The reference's own arithmetic for this op lives in opaque
+ * cubins: parity with its rounding sequence is unpinned. */
+ORACLE_API void oracle_fmha(const void *qkv, const int32_t *seqlens, float *out, int64_t B,
+                            int64_t S, int64_t H, int64_t D, double scale, int causal,
+                            int kind) {
+  const int64_t tok = 3 * H * D;
+#pragma omp parallel
+  {
+    float *q = (float *)malloc((size_t)S * D * sizeof(float));
+    float *k = (float *)malloc((size_t)S * D * sizeof(float));
+    float *v = (float *)malloc((size_t)S * D * sizeof(float));
+    double *p = (double *)malloc((size_t)S * sizeof(double));
+    double *acc = (double *)malloc((size_t)D * sizeof(double));
+#pragma omp for collapse(2) schedule(dynamic)
+    for (int64_t b = 0; b < B; b++) {
+      for (int64_t h = 0; h < H; h++) {
+        int64_t len = seqlens ? (int64_t)seqlens[b] : S;
+        if (len > S) len = S;
+        if (len < 0) len = 0;
+        for (int64_t s = 0; s < S; s++) {
+          const int64_t base = (b * S + s) * tok + h * D;
+          for (int64_t d = 0; d < D; d++) {
+            q[s * D + d] = (float)load_elem(qkv, base + d, kind);
+            k[s * D + d] = (float)load_elem(qkv, base + H * D + d, kind);
+            v[s * D + d] = (float)load_elem(qkv, base + 2 * H * D + d, kind);
+          }
+        }
+        for (int64_t i = 0; i < S; i++) {
+          int64_t nk = len;
+          if (causal && i + 1 < nk) nk = i + 1;
+          float *o = out + (b * S + i) * H * D + h * D;
+          if (nk <= 0) {
+            for (int64_t d = 0; d < D; d++) o[d] = 0.0f;
+            continue;
+          }
+          double mx = -INFINITY;
+          for (int64_t j = 0; j < nk; j++) {
+            double dot = 0.0;
+#pragma omp simd reduction(+ : dot)
+            for (int64_t d = 0; d < D; d++) dot += (double)q[i * D + d] * (double)k[j * D + d];
+            p[j] = dot * scale;
+            if (p[j] > mx) mx = p[j];
+          }
+          double den = 0.0;
+          for (int64_t j = 0; j < nk; j++) {
+            p[j] = exp(p[j] - mx);
+            den += p[j];
+          }
+          for (int64_t d = 0; d < D; d++) acc[d] = 0.0;
+          for (int64_t j = 0; j < nk; j++) {
+            const double pj = p[j];
+#pragma omp simd
+            for (int64_t d = 0; d < D; d++) acc[d] += pj * (double)v[j * D + d];
+          }
+          for (int64_t d = 0; d < D; d++) o[d] = (float)(acc[d] / den);
+        }
+      }
+    }
+    free(q);
+    free(k);
+    free(v);
+    free(p);
+    free(acc);
+  }
+}
+
+/* ------------------------------------------------------------------ */
+/* GEMM with epilogue, casts, QKV transpose                            */
+/* ------------------------------------------------------------------ */
+
+static inline double gelu_erf(double x) { return 0.5 * x * (1.0 + erf(x * 0.70710678118654752440)); }
+
+/* out[M,N] = act(in[M,K] . W[K,N] + bias[N]) + residual[M,N], all row major:
+ * the contract of lib/Kernels/GPU/Ops.cu:134-234 (row-major via the swapped
+ * column-major call at :178-183, bias/ReLU epilogue :152-159, residual through
+ * beta = 1 at :205-209) and of lib/Kernels/CPU/Ops.cpp:34-80.
+ * act: 0 none, 1 ReLU, 2 GELU (exact erf form).
+ * Epilogue order: bias, activation, then residual (the reference adds C after
+ * the epilogue activation; it never combines ReLU with a residual).
+ * Products of the widened inputs are accumulated in fp64.
+ * kind: element type of in / W / bias / residual (0 fp32, 1 fp16, 2 bf16).
+ * pinned by: numpy float64 matmul on the same widened inputs; erf GELU against
+ * scipy.special.erf and torch.nn.functional.gelu. */
+ORACLE_API void oracle_gemm(const void *in, const void *w, const void *bias, const void *residual,
+                            float *out, int64_t M, int64_t N, int64_t K, int act, int kind) {
+  float *wf = (float *)malloc((size_t)K * N * sizeof(float));
+  for (int64_t i = 0; i < K * N; i++) wf[i] = (float)load_elem(w, i, kind);
+#pragma omp parallel
+  {
+    double *row = (double *)malloc((size_t)N * sizeof(double));
+#pragma omp for schedule(static)
+    for (int64_t i = 0; i < M; i++) {
+      for (int64_t j = 0; j < N; j++) row[j] = 0.0;
+      for (int64_t kk = 0; kk < K; kk++) {
+        const double a = load_elem(in, i * K + kk, kind);
+        const float *wr = wf + kk * N;
+#pragma omp simd
+        for (int64_t j = 0; j < N; j++) row[j] += a * (double)wr[j];
+      }
+      for (int64_t j = 0; j < N; j++) {
+        double v = row[j];
+        if (bias) v += load_elem(bias, j, kind);
+        if (act == 1) v = v > 0.0 ? v : 0.0;
+        if (act == 2) v = gelu_erf(v);
+        if (residual) v += load_elem(residual, i * N + j, kind);
+        out[i * N + j] = (float)v;
+      }
+    }
+    free(row);
+  }
+  free(wf);
+}
+
+/* fp32 -> fp16 bits, round to nearest even (lib/Kernels/GPU/Utils.cu:16-83:
+ * __float2half / __float22half2_rn). pinned by numpy astype(float16). */
+ORACLE_API void oracle_cast_f32_to_f16(const float *src, uint16_t *dst, int64_t n) {
+  for (int64_t i = 0; i < n; i++) dst[i] = double_to_half_bits((double)src[i]);
+}
+
+/* [token, 3, H, D] + bias[3, H, D] -> q, k, v each [B, H, S, D]
+ * (lib/Kernels/GPU/Transpose.cu:5-51).  Sum in fp32, rounded to kind.
+ * pinned by: numpy reshape/transpose of the same arrays. */
+ORACLE_API void oracle_qkv_bias_transpose(const void *qkv, const void *bias, float *q, float *k,
+                                          float *v, int64_t B, int64_t S, int64_t H, int64_t D,
+                                          int kind) {
+  float *dst[3] = {q, k, v};
+  for (int64_t b = 0; b < B; b++)
+    for (int64_t s = 0; s < S; s++)
+      for (int64_t w = 0; w < 3; w++)
+        for (int64_t h = 0; h < H; h++)
+          for (int64_t d = 0; d < D; d++) {
+            float x = (float)load_elem(qkv, (((b * S + s) * 3 + w) * H + h) * D + d, kind);
+            if (bias) x += (float)load_elem(bias, (w * H + h) * D + d, kind);
+            dst[w][((b * H + h) * S + s) * D + d] = (float)round_to_kind((double)x, kind);
+          }
+}
+
+/* ------------------------------------------------------------------ */
+/* Encoder layers (composition)                                        */
+/* ------------------------------------------------------------------ */
+
+static uint16_t *to_half_buf(const float *src, int64_t n) {
+  uint16_t *dst = (uint16_t *)malloc((size_t)n * sizeof(uint16_t));
+  for (int64_t i = 0; i < n; i++) dst[i] = double_to_half_bits((double)src[i]);
+  return dst;
+}
+
+/* Pre-LN transformer layer with the dataflow of lib/Kernels/GPU/LLM.cu:26-159
+ * (CPU twin lib/Kernels/CPU/LLM.cpp:191-383):
+ *   xh  = fp16(x)                                   (LLM.cu:35-37)
+ *   a   = LN(xh)              gamma = 1, beta = 0   (:40-52)
+ *   qkv = a . Wqkv            [M, 3d] = [B,S,3,H,Dh](:70-72, LLM.cpp:243-246)
+ *   ctx = fMHA(qkv)           scale 1/sqrt(Dh), causal flag (:79-81)
+ *   pr  = ctx . Wo + bo                             (:95-97)
+ *   y   = pr + xh ; n2 = LN(y)                      (:112-114)
+ *   f   = act(n2 . W1 + b1)                         (:119-121)
+ *   out = fp32(f . W2 + b2 + y)                     (:136-141)
+ * All weights arrive as fp32 and are rounded to fp16 first (:55-57,84-90,
+ * 100-106,124-130); every tensor that the GPU path keeps in fp16 is rounded to
+ * fp16 here at the same place, everything between two roundings is fp64.
+ * Deliberate, documented departures from the reference's GPU body: head_num,
+ * is_casual and is_relu are honoured (the reference ignores them and
+ * hard-wires 8 x 128 heads, causal, ReLU - LLM.cu:18-19,79-81,119-121) and
+ * GEMMs accumulate in >= fp32 (the reference asks for fp16 accumulation,
+ * Ops.cu:164-167, whose results only a CUDA run could pin).
+ * act: 1 ReLU, 2 GELU(erf).
+ * pinned by: composition of the pinned pieces above; cross-checked against a
+ * torch fp64 restatement in the tests.  Parity with the reference's own
+ * rounding sequence is unpinned (cuBLASLt fp16 accumulate, cubin attention). */
+ORACLE_API void oracle_decoding_context_layer(const float *input, const float *wqkv,
+                                              const float *wo, const float *bo, const float *w1,
+                                              const float *b1, const float *w2, const float *b2,
+                                              float *output, int64_t B, int64_t S, int64_t d,
+                                              int64_t ffn, int64_t H, int causal, int act) {
+  const int64_t M = B * S, Dh = d / H;
+  uint16_t *xh = to_half_buf(input, M * d);
+  uint16_t *wqkv_h = to_half_buf(wqkv, d * 3 * d);
+  uint16_t *wo_h = to_half_buf(wo, d * d), *bo_h = to_half_buf(bo, d);
+  uint16_t *w1_h = to_half_buf(w1, d * ffn), *b1_h = to_half_buf(b1, ffn);
+  uint16_t *w2_h = to_half_buf(w2, ffn * d), *b2_h = to_half_buf(b2, d);
+  float *t0 = (float *)malloc((size_t)M * d * sizeof(float));
+  float *t1 = (float *)malloc((size_t)M * 3 * d * sizeof(float));
+  float *t2 = (float *)malloc((size_t)M * ffn * sizeof(float));
+
+  oracle_layernorm(xh, NULL, NULL, t0, 1e-5, M, d, 1);
+  uint16_t *a_h = to_half_buf(t0, M * d);
+  oracle_gemm(a_h, wqkv_h, NULL, NULL, t1, M, 3 * d, d, 0, 1);
+  uint16_t *qkv_h = to_half_buf(t1, M * 3 * d);
+  oracle_fmha(qkv_h, NULL, t0, B, S, H, Dh, 1.0 / sqrt((double)Dh), causal, 1);
+  uint16_t *ctx_h = to_half_buf(t0, M * d);
+  oracle_gemm(ctx_h, wo_h, bo_h, NULL, t0, M, d, d, 0, 1);
+  uint16_t *pr_h = to_half_buf(t0, M * d);
+  float *ysum = (float *)malloc((size_t)M * d * sizeof(float));
+  oracle_add_residual_layernorm(pr_h, xh, NULL, NULL, ysum, t0, 1e-5, M, d, 1);
+  uint16_t *y_h = to_half_buf(ysum, M * d);
+  uint16_t *n2_h = to_half_buf(t0, M * d);
+  oracle_gemm(n2_h, w1_h, b1_h, NULL, t2, M, ffn, d, act, 1);
+  uint16_t *f_h = to_half_buf(t2, M * ffn);
+  oracle_gemm(f_h, w2_h, b2_h, y_h, t0, M, d, ffn, 0, 1);
+  for (int64_t i = 0; i < M * d; i++)
+    output[i] = half_bits_to_float(double_to_half_bits((double)t0[i]));
+
+  free(xh); free(wqkv_h); free(wo_h); free(bo_h); free(w1_h); free(b1_h); free(w2_h); free(b2_h);
+  free(t0); free(t1); free(t2); free(a_h); free(qkv_h); free(ctx_h); free(pr_h); free(ysum);
+  free(y_h); free(n2_h); free(f_h);
+}
+
+/* Post-LN BERT-base encoder layer on fp16 tensors (the benchmark's fifth
+ * configuration; its ordering and GELU are defined by that configuration, not
+ * by the reference, whose layer is the pre-LN one above):
+ *   qkv = x . Wqkv + bqkv          [M, 3d] read as [B,S,3,H,Dh]
+ *   ctx = fMHA(qkv, seqlens)       scale 1/sqrt(Dh), no causal mask
+ *   h1  = LN1(ctx . Wo + bo + x)   gamma1, beta1
+ *   f   = GELU_erf(h1 . W1 + b1)
+ *   out = LN2(f . W2 + b2 + h1)    gamma2, beta2
+ * All tensors fp16 bits; intermediates are rounded to fp16 where the GPU path
+ * stores them; out is returned un-rounded in fp32.
+ * pinned by: composition of pinned pieces; torch fp64 restatement in tests. */
+ORACLE_API void oracle_bert_layer_f16(const uint16_t *x, const uint16_t *wqkv, const uint16_t *bqkv,
+                                      const uint16_t *wo, const uint16_t *bo, const uint16_t *g1,
+                                      const uint16_t *be1, const uint16_t *w1, const uint16_t *b1,
+                                      const uint16_t *w2, const uint16_t *b2, const uint16_t *g2,
+                                      const uint16_t *be2, const int32_t *seqlens, float *out,
+                                      int64_t B, int64_t S, int64_t d, int64_t ffn, int64_t H,
+                                      double eps) {
+  const int64_t M = B * S, Dh = d / H;
+  float *t0 = (float *)malloc((size_t)M * d * sizeof(float));
+  float *t1 = (float *)malloc((size_t)M * 3 * d * sizeof(float));
+  float *t2 = (float *)malloc((size_t)M * ffn * sizeof(float));
+  float *sum = (float *)malloc((size_t)M * d * sizeof(float));
+
+  oracle_gemm(x, wqkv, bqkv, NULL, t1, M, 3 * d, d, 0, 1);
+  uint16_t *qkv_h = to_half_buf(t1, M * 3 * d);
+  oracle_fmha(qkv_h, seqlens, t0, B, S, H, Dh, 1.0 / sqrt((double)Dh), 0, 1);
+  uint16_t *ctx_h = to_half_buf(t0, M * d);
+  oracle_gemm(ctx_h, wo, bo, NULL, t0, M, d, d, 0, 1);
+  uint16_t *pr_h = to_half_buf(t0, M * d);
+  oracle_add_residual_layernorm(pr_h, x, g1, be1, sum, t0, eps, M, d, 1);
+  uint16_t *h1_h = to_half_buf(t0, M * d);
+  oracle_gemm(h1_h, w1, b1, NULL, t2, M, ffn, d, 2, 1);
+  uint16_t *f_h = to_half_buf(t2, M * ffn);
+  oracle_gemm(f_h, w2, b2, NULL, t0, M, d, ffn, 0, 1);
+  uint16_t *o_h = to_half_buf(t0, M * d);
+  oracle_add_residual_layernorm(o_h, h1_h, g2, be2, sum, out, eps, M, d, 1);
+
+  free(t0); free(t1); free(t2); free(sum); free(qkv_h); free(ctx_h); free(pr_h); free(h1_h);
+  free(f_h); free(o_h);
+}
