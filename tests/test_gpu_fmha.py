@@ -1,0 +1,127 @@
+"""Parity of the HIP fused multi-head attention (C ABI mgpuFusedMHAF16 / BF16)
+with the oracle: max absolute error <= 2e-3 on fp16 outputs against the fp32/64
+CPU result (bf16: <= 8e-3, its output spacing below 1 being 2^-8)."""
+import numpy as np
+import pytest
+
+from conftest import to_dev
+
+pytestmark = pytest.mark.gpu
+
+TOL_F16 = 2e-3
+TOL_BF16 = 8e-3
+
+
+def run(pkg, gpu, qkv, lens=None, causal=False, scale=None):
+    tl = to_dev(np.asarray(lens, np.int32), gpu) if lens is not None else None
+    return pkg.fused_mha(to_dev(qkv, gpu), tl, scale=scale, causal=causal).cpu().numpy().astype(np.float32)
+
+
+def make_qkv(rng, B, S, H, std=1.0 / 8):
+    return (rng.standard_normal((B, S, 3, H, 64)) * std).astype(np.float16)
+
+
+def test_fmha_config2_b32_s128_h12(pkg, gpu, oracle):
+    rng = np.random.Generator(np.random.PCG64(20242))
+    qkv = make_qkv(rng, 32, 128, 12)
+    got = run(pkg, gpu, qkv)
+    assert np.abs(got - oracle.fmha(qkv)).max() <= TOL_F16
+
+
+def test_fmha_config3_b8_s512_h16_key_padding(pkg, gpu, oracle):
+    rng = np.random.Generator(np.random.PCG64(20243))
+    qkv = make_qkv(rng, 8, 512, 16)
+    lens = rng.integers(256, 513, 8).astype(np.int32)
+    got = run(pkg, gpu, qkv, lens)
+    assert np.abs(got - oracle.fmha(qkv, lens)).max() <= TOL_F16
+
+
+def test_fmha_roofline_shape_b32_s512_h12(pkg, gpu, oracle):
+    rng = np.random.Generator(np.random.PCG64(20244))
+    qkv = make_qkv(rng, 32, 512, 12)
+    got = run(pkg, gpu, qkv)
+    assert np.abs(got - oracle.fmha(qkv)).max() <= TOL_F16
+
+
+# ragged S (partial query blocks and partial key tiles), S below one tile,
+# lengths of 0 / 1 / exactly on and one past a tile boundary
+@pytest.mark.parametrize("B,S,H,lens", [
+    (1, 1, 1, None), (2, 5, 2, None), (1, 63, 1, None), (1, 64, 2, None), (1, 65, 1, None),
+    (2, 127, 3, None), (1, 129, 2, None), (2, 200, 3, [1, 150]), (3, 192, 2, [64, 65, 128]),
+    (2, 300, 1, [300, 299]), (4, 96, 2, [0, 1, 2, 96]), (1, 1000, 1, [777]), (2, 128, 4, [500, -3]),
+])
+def test_fmha_ragged_and_masked(pkg, gpu, oracle, rng, B, S, H, lens):
+    qkv = make_qkv(rng, B, S, H)
+    got = run(pkg, gpu, qkv, lens)
+    ref = oracle.fmha(qkv, lens)
+    assert np.abs(got - ref).max() <= TOL_F16
+    if lens is not None:
+        for b, l in enumerate(lens):
+            if l <= 0:
+                assert np.all(got[b] == 0)  # no admissible key -> zeros
+
+
+@pytest.mark.parametrize("B,S,H,lens", [(2, 128, 2, None), (1, 257, 2, None), (2, 512, 1, [512, 100]),
+                                        (1, 70, 3, [33])])
+def test_fmha_causal(pkg, gpu, oracle, rng, B, S, H, lens):
+    qkv = make_qkv(rng, B, S, H)
+    got = run(pkg, gpu, qkv, lens, causal=True)
+    assert np.abs(got - oracle.fmha(qkv, lens, causal=True)).max() <= TOL_F16
+
+
+def test_fmha_large_logits_and_other_scales(pkg, gpu, oracle, rng):
+    """Peaked softmax rows (|logit| up to ~60) exercise the running-maximum
+    rescaling; the scale is a free parameter of the entry point."""
+    qkv = make_qkv(rng, 2, 256, 2, std=1.0)
+    for scale in (0.125, 1.0, 0.01):
+        got = run(pkg, gpu, qkv, scale=scale)
+        assert np.abs(got - oracle.fmha(qkv, scale=scale)).max() <= 4e-3 if scale == 1.0 else TOL_F16
+
+
+def test_fmha_padding_garbage_is_ignored(pkg, gpu, oracle, rng):
+    """Keys past the valid length may hold anything, NaN and Inf included."""
+    qkv = make_qkv(rng, 2, 160, 2)
+    lens = [100, 37]
+    ref = oracle.fmha(qkv, lens)
+    dirty = qkv.copy()
+    for b, l in enumerate(lens):
+        dirty[b, l:, 1:] = np.float16(np.nan)
+        dirty[b, l::2, 1:] = np.float16(np.inf)
+    got = run(pkg, gpu, dirty, lens)
+    assert np.isfinite(got).all() and np.abs(got - ref).max() <= TOL_F16
+
+
+def test_fmha_identities_at_full_size(pkg, gpu):
+    """Size-independent properties at the roofline shape (b32 s512 h12):
+    constant V gives that constant, Q = 0 gives the mean of V, permuting the
+    keys (K and V rows together) changes nothing beyond rounding."""
+    import torch
+    g = torch.Generator(device=gpu)
+    g.manual_seed(11)
+    B, S, H = 32, 512, 12
+    qkv = (torch.randn((B, S, 3, H, 64), device=gpu, generator=g) / 8).half()
+    base = pkg.fused_mha(qkv).float()
+    c = qkv.clone()
+    c[:, :, 2] = 0.375
+    assert (pkg.fused_mha(c).float() - 0.375).abs().max().item() <= 1e-3
+    z = qkv.clone()
+    z[:, :, 0] = 0
+    mean_v = z[:, :, 2].float().mean(1).reshape(B, 1, H * 64)
+    assert (pkg.fused_mha(z).float() - mean_v).abs().max().item() <= 1e-3
+    perm = torch.randperm(S, device=gpu, generator=g)
+    p = qkv.clone()
+    p[:, :, 1:] = qkv[:, perm, 1:]
+    assert (pkg.fused_mha(p).float() - base).abs().max().item() <= 1e-3
+    assert torch.equal(pkg.fused_mha(qkv), pkg.fused_mha(qkv))  # deterministic
+
+
+def test_fmha_bf16(pkg, gpu, oracle, rng):
+    import torch
+    for (B, S, H, lens, causal) in [(2, 128, 2, None, False), (2, 200, 3, [200, 77], False), (1, 130, 1, None, True)]:
+        f = (rng.standard_normal((B, S, 3, H, 64)) / 8).astype(np.float32)
+        t = torch.from_numpy(f).to(gpu).to(torch.bfloat16)
+        tl = to_dev(np.asarray(lens, np.int32), gpu) if lens is not None else None
+        got = pkg.fused_mha(t, tl, causal=causal).float().cpu().numpy()
+        bits = t.view(torch.int16).cpu().numpy().view(np.uint16)
+        ref = oracle.fmha(bits, lens, causal=causal, bf16=True)
+        assert np.abs(got - ref).max() <= TOL_BF16

@@ -1,0 +1,114 @@
+"""Casts, QKV bias+transpose, GEMM epilogues and the two layer entry points
+against the oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+from conftest import to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n", [1, 7, 8, 9, 1000, 65537, 3 * 768 * 768])
+def test_casts_bit_exact(pkg, gpu, oracle, rng, n):
+    f = (rng.standard_normal(n) * np.exp(rng.uniform(-20, 12, n))).astype(np.float32)
+    h = pkg.cast_f32_to_f16(to_dev(f, gpu))
+    assert np.array_equal(h.cpu().numpy().view(np.uint16), oracle.cast_f32_to_f16(f).view(np.uint16))
+    back = pkg.cast_f16_to_f32(h).cpu().numpy()
+    assert np.array_equal(back.view(np.uint32), oracle.half_to_float(h.cpu().numpy()).view(np.uint32))
+
+
+def test_cast_special_values(pkg, gpu, oracle):
+    f = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 65504.0, 65520.0, 65519.9, 1e-8, 5.96e-8, 2.98e-8,
+                  2.99e-8, 6.1e-5, 1.0 + 2 ** -11, 1.0 + 2 ** -11 + 2 ** -20, 1.0 + 3 * 2 ** -11], np.float32)
+    h = pkg.cast_f32_to_f16(to_dev(f, gpu)).cpu().numpy()
+    ref = oracle.cast_f32_to_f16(f)
+    assert np.all((h.view(np.uint16) == ref.view(np.uint16)) | (np.isnan(h) & np.isnan(ref)))
+
+
+def test_qkv_bias_transpose(pkg, gpu, oracle, rng):
+    B, S, H, D = 3, 50, 4, 64
+    qkv = rng.standard_normal((B, S, 3, H, D)).astype(np.float16)
+    bias = rng.standard_normal((3, H, D)).astype(np.float16)
+    t = to_dev(qkv, gpu)
+    q, k, v = pkg.qkv_bias_transpose(t, to_dev(bias, gpu))
+    rq, rk, rv = oracle.qkv_bias_transpose(qkv, bias)
+    for got, ref in ((q, rq), (k, rk), (v, rv)):
+        assert np.array_equal(got.cpu().numpy().astype(np.float32), ref)
+    # the packed tensor is updated in place with the bias, like the reference kernel
+    upd = (qkv.astype(np.float32) + bias.astype(np.float32)[None, None]).astype(np.float16)
+    assert np.array_equal(t.cpu().numpy(), upd)
+
+
+def f16_tol(ref, k_ulp=1.0, floor=1e-3):
+    e = np.floor(np.log2(np.maximum(np.abs(ref), 2.0 ** -14)))
+    return k_ulp * 2.0 ** (e - 10) + floor
+
+
+@pytest.mark.parametrize("M,K,N", [(512, 768, 2304), (100, 64, 72), (4096, 3072, 768), (33, 128, 8)])
+def test_matmul_ex_f16_epilogues(pkg, gpu, oracle, rng, M, K, N):
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    b = rng.standard_normal(N).astype(np.float16)
+    r = rng.standard_normal((M, N)).astype(np.float16)
+    tx, tw, tb, tr = [to_dev(t, gpu) for t in (x, w, b, r)]
+    for kw, okw in [(dict(), dict()), (dict(bias=tb), dict(bias=b)),
+                    (dict(bias=tb, act=pkg.ACT_RELU), dict(bias=b, act=oracle.ACT_RELU)),
+                    (dict(bias=tb, act=pkg.ACT_GELU), dict(bias=b, act=oracle.ACT_GELU)),
+                    (dict(bias=tb, residual=tr), dict(bias=b, residual=r))]:
+        got = pkg.matmul_ex(tx, tw, **kw).cpu().numpy().astype(np.float32)
+        ref = oracle.gemm(x, w, **okw)
+        assert np.all(np.abs(got - ref) <= f16_tol(ref)), (kw.keys(), np.abs(got - ref).max())
+
+
+def test_matmul_f32(pkg, gpu, oracle, rng):
+    M, K, N = 200, 96, 130
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    got = pkg.matmul_ex(to_dev(x, gpu), to_dev(w, gpu), to_dev(b, gpu)).cpu().numpy()
+    ref = oracle.gemm(x, w, b)
+    # fp32 GEMM on the matrix cores may use reduced-precision products
+    assert np.abs(got - ref).max() <= 2e-2
+    assert np.abs(got - ref).mean() <= 2e-3
+
+
+def layer_tol(ref):
+    """fp16 output of an O(1..4)-magnitude tensor after ~6 fp16-rounded stages."""
+    return 2e-3 + 4e-3 * np.abs(ref)
+
+
+def test_bert_encoder_layer_config4(pkg, gpu, oracle):
+    """BERT-base layer (32,128,768) fp16, weights N(0, 0.02): post-LN ordering
+    and erf-GELU are defined by the benchmark configuration, not by the
+    reference (whose layer is pre-LN / ReLU / causal)."""
+    rng = np.random.Generator(np.random.PCG64(20245))
+    B, S, d, ffn, H = 32, 128, 768, 3072, 12
+    h16 = lambda *s: (0.02 * rng.standard_normal(s)).astype(np.float16)
+    gam = lambda: (1 + 0.02 * rng.standard_normal(d)).astype(np.float16)
+    x = rng.standard_normal((B, S, d)).astype(np.float16)
+    P = [h16(d, 3 * d), h16(3 * d), h16(d, d), h16(d), gam(), h16(d), h16(d, ffn), h16(ffn), h16(ffn, d),
+         h16(d), gam(), h16(d)]
+    for lens in (None, rng.integers(1, 129, B).astype(np.int32)):
+        tl = to_dev(lens, gpu) if lens is not None else None
+        got = pkg.bert_encoder_layer(to_dev(x, gpu), *[to_dev(p, gpu) for p in P], heads=H, seqlens=tl)
+        got = got.cpu().numpy().astype(np.float32)
+        ref = oracle.bert_layer_f16(x, *P, heads=H, seqlens=lens)
+        err = np.abs(got - ref)
+        assert np.all(err <= layer_tol(ref)), err.max()
+        assert err.mean() <= 5e-4
+
+
+@pytest.mark.parametrize("causal,relu", [(True, True), (False, False)])
+def test_decoding_context_layer(pkg, gpu, oracle, rng, causal, relu):
+    B, S, d, ffn, H = 4, 128, 512, 2048, 8
+    f = lambda *s, sc=0.03: (sc * rng.standard_normal(s)).astype(np.float32)
+    x = rng.standard_normal((B, S, d)).astype(np.float32)
+    W = [f(d, 3 * d), f(d, d), f(d), f(d, ffn), f(ffn), f(ffn, d), f(d)]
+    got = pkg.decoding_context_layer(to_dev(x, gpu), *[to_dev(w, gpu) for w in W], heads=H, causal=causal,
+                                     relu=relu).cpu().numpy()
+    ref = oracle.decoding_context_layer(x, *W, heads=H, causal=causal,
+                                        act=oracle.ACT_RELU if relu else oracle.ACT_GELU)
+    err = np.abs(got - ref)
+    assert np.all(err <= layer_tol(ref)), err.max()
+    # output is fp16-representable fp32, like the reference's final cast
+    assert np.array_equal(got, got.astype(np.float16).astype(np.float32))
