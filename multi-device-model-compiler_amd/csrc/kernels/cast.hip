@@ -23,8 +23,8 @@ __global__ __launch_bounds__(256) void cast_f32_to_f16_vec8_kernel(f16x8 *__rest
                                                                    size_t n8) {
   const size_t stride = (size_t)gridDim.x * 256;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += stride) {
-    const f32x4 lo = __builtin_nontemporal_load(src + 2 * i);
-    const f32x4 hi = __builtin_nontemporal_load(src + 2 * i + 1);
+    const f32x4 lo = src[2 * i];
+    const f32x4 hi = src[2 * i + 1];
     f16x8 o;
 #pragma unroll
     for (int e = 0; e < 4; e++) {
@@ -40,7 +40,7 @@ __global__ __launch_bounds__(256) void cast_f16_to_f32_vec8_kernel(f32x4 *__rest
                                                                    size_t n8) {
   const size_t stride = (size_t)gridDim.x * 256;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += stride) {
-    const f16x8 v = __builtin_nontemporal_load(src + i);
+    const f16x8 v = src[i];
     f32x4 lo, hi;
 #pragma unroll
     for (int e = 0; e < 4; e++) {

@@ -9,9 +9,10 @@
 //
 // Work decomposition.  A 256-thread block (4 wavefronts) owns BM = 128 * NQ
 // consecutive queries of one (batch, head); each wavefront owns NQ blocks of 32
-// queries.  Key/value tiles of BN = 64 keys are staged through LDS (double
-// buffered, next tile's global loads in flight while the current one is
-// consumed) and shared by the 4 wavefronts.
+// queries.  Key/value tiles of BN = 64 keys travel HBM -> LDS directly
+// (global_load_lds, 16 bytes per lane, no register staging) into a ring of
+// three LDS stages shared by the 4 wavefronts, so two tiles are always in
+// flight behind the one being consumed.
 //
 // MFMA formulation (v_mfma_f32_32x32x16_{f16,bf16}; operand lane layout: lane l
 // supplies row/col l%32 and k-slots 8*(l/32)..+7; the 32x32 accumulator gives
@@ -26,11 +27,35 @@
 //     and the contraction over keys does not care in which k-slot a key sits as
 //     long as the A operand (V^T) is read with the same assignment - two 8-byte
 //     LDS reads per operand.  P never leaves registers.
-// V is transposed on its way into LDS (4x4 halves in registers, 8-byte writes),
-// rows padded so that operand reads are bank-conflict free.
+// Both tiles sit in LDS row-major as in memory (64 rows of 128 bytes).  The
+// direct loads write 1 KiB of consecutive LDS per wavefront instruction, so
+// rows cannot be padded; instead each lane fetches the 16-byte chunk
+// c ^ swizzle(row) of its row, which makes the K operand reads (ds_read_b128,
+// 16 rows per cycle) and the V operand reads conflict free.  V^T operands come
+// from ds_read_b64_tr_b16, the transposing LDS read of gfx950: within 16
+// lanes, lane L receives element L%4 of the four 8-byte rows addressed by
+// lanes L/4, L/4+4, L/4+8, L/4+12 - four keys of one d column.
 //
-// Softmax runs in fp32 in base 2: p = exp2(s*c - m*c), c = scale*log2(e), with
-// the usual running maximum / running sum rescaling.
+// Softmax runs in fp32 in base 2.  At head_dim 64 the softmax VALU work per
+// score costs about as many issue cycles as the 256 MFMA flops that score pays
+// for, so the loop is trimmed to exp2 + half a max3 + half a convert + half a
+// dot2 per score:
+//   * Q is multiplied by c = scale*log2(e) once (rounded to the 16-bit type: a
+//     relative perturbation of at most half an ulp of Q), and the running
+//     offset m is subtracted BY THE MATRIX CORE: the first MFMA of each score
+//     block takes a register block holding -m as its C operand, so the scores
+//     come out as s*c - m and need no VALU fma;
+//   * m is the row maximum as of the last adjustment, not of the current tile:
+//     it is only advanced (and O, l rescaled, the -m block rewritten) when some
+//     row of the wavefront sees a score more than 2^8 above it.  p stays <= 256,
+//     well inside fp16, and O / l is unchanged because both use the same m;
+//   * the row sum is taken with v_dot2_f32_{f16,bf16} over the already converted
+//     P pairs (two scores per instruction; the normaliser then matches the P
+//     the matrix cores consume);
+//   * accumulators stay in VGPRs (two wavefronts per SIMD leave 256 registers
+//     each, so no AGPR copies).
+// The output tile is transposed through LDS so that every store instruction
+// writes whole 128-byte rows.
 #include "common.hpp"
 #include "mgpu_ops_internal.hpp"
 #include "types.hpp"
@@ -45,11 +70,14 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kD = 64;   // head dim
 constexpr int kBN = 64;  // keys per tile
-constexpr int kKS = 72;  // K tile row stride in elements (144 B: conflict-free 16 B reads)
-constexpr int kVS = 68;  // V^T tile row stride in elements (136 B: conflict-free 8 B reads)
+constexpr int kStages = 3;               // LDS ring depth
+constexpr int kTileBytes = kBN * kD * 2; // one K or V tile: 64 rows of 128 B, unpadded
+constexpr int kOS = 68;  // output staging row stride in elements
+constexpr float kLazyLog2 = 8.0f; // re-centre only when a score exceeds the offset by 2^8
 
 template <typename T> struct Mma;
 template <> struct Mma<_Float16> {
@@ -59,6 +87,17 @@ template <> struct Mma<_Float16> {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
   __device__ static __forceinline__ _Float16 narrow(float f) { return (_Float16)f; }
+  __device__ static __forceinline__ float widen(_Float16 h) { return (float)h; }
+  __device__ static __forceinline__ v4 readTr(const unsigned char *p) {
+    return __builtin_bit_cast(v4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 __attribute__((address_space(3))) *)p));
+  }
+  // acc + sum of the two packed values of word w of a v8
+  __device__ static __forceinline__ float pairSum(v8 p, int w, float acc) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const h2 pair = {p[2 * w], p[2 * w + 1]};
+    const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(pair, ones, acc, false);
+  }
 };
 template <> struct Mma<bf16_t> {
   using v8 = bf16x8;
@@ -67,6 +106,16 @@ template <> struct Mma<bf16_t> {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
   __device__ static __forceinline__ __bf16 narrow(float f) { return (__bf16)f; }
+  __device__ static __forceinline__ float widen(__bf16 h) { return (float)h; }
+  __device__ static __forceinline__ v4 readTr(const unsigned char *p) {
+    return __builtin_bit_cast(v4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 __attribute__((address_space(3))) *)p));
+  }
+  __device__ static __forceinline__ float pairSum(v8 p, int w, float acc) {
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    const b2 pair = {p[2 * w], p[2 * w + 1]};
+    const b2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(pair, ones, acc, false);
+  }
 };
 
 // Exchange with lane l ^ 32: v_permlane32_swap hands every lane the value of
@@ -83,17 +132,18 @@ __device__ __forceinline__ float halves_sum(float v) {
 }
 
 template <typename T, int NQ, bool CAUSAL>
-__global__ __launch_bounds__(256) void fmha_fwd_d64_kernel(const uint16_t *__restrict__ qkv,
-                                                           const int32_t *__restrict__ seqlens,
-                                                           uint16_t *__restrict__ out, int S, int H,
-                                                           int nQB, float scale_log2e) {
+__global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__restrict__ qkv,
+                                                              const int32_t *__restrict__ seqlens,
+                                                              uint16_t *__restrict__ out, int S, int H,
+                                                              int nQB, float scale_log2e) {
   using M = Mma<T>;
   using v8 = typename M::v8;
   using v4 = typename M::v4;
   constexpr int BM = 128 * NQ;
 
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][kBN * kKS];
-  __shared__ __attribute__((aligned(16))) uint16_t Vt[2][kD * kVS];
+  // Ring of kStages stages, each a K tile followed by a V tile; reused as the
+  // output staging area at the end.
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[kStages * 2 * kTileBytes];
 
   // Work-item order: query blocks of one (batch, head) are consecutive, and a
   // contiguous run of work items goes to each of the 8 XCDs (consecutive block
@@ -109,7 +159,7 @@ __global__ __launch_bounds__(256) void fmha_fwd_d64_kernel(const uint16_t *__res
 
   const int tid = threadIdx.x;
   const int lane = tid % 64;
-  const int wave = tid / 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int l32 = lane % 32;
   const int hl = lane / 32;
 
@@ -119,21 +169,10 @@ __global__ __launch_bounds__(256) void fmha_fwd_d64_kernel(const uint16_t *__res
     kvlen = kvlen < 0 ? 0 : (kvlen > S ? S : kvlen);
   }
   const int q0 = qb * BM + wave * (NQ * 32); // first query of this wavefront
-  const size_t tok = (size_t)3 * H * kD;      // elements per token row
-  const uint16_t *qbase = qkv + (size_t)b * S * tok + (size_t)h * kD;
-  const uint16_t *kbase = qbase + (size_t)H * kD;
-  const uint16_t *vbase = qbase + (size_t)2 * H * kD;
-
-  // Q as the B operand: lane (query l32, k-slots = d 16c + 8hl .. +7).
-  v8 qf[NQ][4];
-#pragma unroll
-  for (int qi = 0; qi < NQ; qi++) {
-    int row = q0 + qi * 32 + l32;
-    row = row < S ? row : S - 1;
-#pragma unroll
-    for (int c = 0; c < 4; c++)
-      qf[qi][c] = *reinterpret_cast<const v8 *>(qbase + (size_t)row * tok + 16 * c + 8 * hl);
-  }
+  const uint32_t tokBytes = (uint32_t)3 * H * kD * 2; // bytes per token row
+  const char *qbase = reinterpret_cast<const char *>(qkv) + ((size_t)b * S * 3 * H + h) * kD * 2;
+  const char *kbase = qbase + (size_t)H * kD * 2;
+  const char *vbase = qbase + (size_t)2 * H * kD * 2;
 
   int kend = kvlen;
   if (CAUSAL) {
@@ -143,87 +182,143 @@ __global__ __launch_bounds__(256) void fmha_fwd_d64_kernel(const uint16_t *__res
   }
   const int nkt = (kend + kBN - 1) / kBN;
 
-  // Tile movers.  K: thread -> rows tid/8 and tid/8 + 32, 8 elements at
-  // column 8*(tid%8).  V: thread -> rows 4*(tid/16)..+3, 4 elements at column
-  // 4*(tid%16), transposed in registers before the LDS write.
-  const int krow = tid / 8, kcol = (tid % 8) * 8;
-  const int vk0 = 4 * (tid / 16), vd0 = 4 * (tid % 16);
-  u32x4 kreg[2];
-  u32x2 vreg[4];
-
-  auto loadTile = [&](int kt) {
+  // ---- tile movers: HBM -> LDS, 16 bytes per lane ---------------------------
+  // One wavefront instruction fills 1 KiB = 8 tile rows; wavefront w moves rows
+  // 16w .. 16w+15 of both tiles.  Lane l lands in LDS chunk l%8 of row l/8 and
+  // fetches global chunk (l%8) ^ swizzle(row): swizzle = (row/2)%8 for K,
+  // 4*((row/2)%2) for V.
+  const int mrow = lane / 8, mchunk = lane % 8;
+  uint32_t koff[2], voff[2];
 #pragma unroll
-    for (int r = 0; r < 2; r++) {
-      int key = kt * kBN + krow + 32 * r;
-      key = key < S ? key : S - 1;
-      kreg[r] = *reinterpret_cast<const u32x4 *>(kbase + (size_t)key * tok + kcol);
-    }
+  for (int i = 0; i < 2; i++) {
+    const int row = 8 * (2 * wave + i) + mrow;
+    koff[i] = (uint32_t)row * tokBytes + (uint32_t)((mchunk ^ ((row >> 1) & 7)) * 16);
+    voff[i] = (uint32_t)row * tokBytes + (uint32_t)((mchunk ^ (((row >> 1) & 1) << 2)) * 16);
+  }
+  // The loads are written as inline assembly so that the compiler's wait-count
+  // bookkeeping does not see them: it would otherwise wait for every load in
+  // flight, prefetches included, before any later LDS read.  Completion is
+  // tracked by hand with s_waitcnt vmcnt(n) below (4 loads per tile and wave).
+  const uint32_t ldsBase = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) unsigned char *)smem);
+  auto dma16 = [&](uint32_t voffset, const char *sbase, uint32_t ldsAddr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voffset), "s"(sbase), "s"(ldsAddr)
+                 : "memory");
+  };
+  auto issueTile = [&](int kt) {
+    const uint32_t kdst = ldsBase + (uint32_t)((kt % kStages) * (2 * kTileBytes) + (2 * wave) * 1024);
+    const uint32_t vdst = kdst + kTileBytes;
+    if (kt * kBN + kBN <= S) { // whole tile inside the sequence
+      const char *kg = kbase + (size_t)kt * kBN * tokBytes;
+      const char *vg = vbase + (size_t)kt * kBN * tokBytes;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int key = kt * kBN + vk0 + i;
-      const int keyc = key < S ? key : S - 1;
-      u32x2 v = *reinterpret_cast<const u32x2 *>(vbase + (size_t)keyc * tok + vd0);
-      // Rows of masked keys meet p = 0; zero them so that stray NaN/Inf bits in
-      // padding cannot reach the accumulators.
-      if (key >= kvlen) v = u32x2{0u, 0u};
-      vreg[i] = v;
+      for (int i = 0; i < 2; i++) {
+        dma16(koff[i], kg, kdst + i * 1024);
+        dma16(voff[i], vg, vdst + i * 1024);
+      }
+    } else { // last tile of a ragged sequence: clamp the row, the mask hides it
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        const int row = 8 * (2 * wave + i) + mrow;
+        int key = kt * kBN + row;
+        key = key < S ? key : S - 1;
+        const uint32_t rowBytes = (uint32_t)key * tokBytes;
+        dma16(rowBytes + (mchunk ^ ((row >> 1) & 7)) * 16, kbase, kdst + i * 1024);
+        dma16(rowBytes + (mchunk ^ (((row >> 1) & 1) << 2)) * 16, vbase, vdst + i * 1024);
+      }
     }
   };
-  auto storeTile = [&](int buf) {
-#pragma unroll
-    for (int r = 0; r < 2; r++)
-      *reinterpret_cast<u32x4 *>(&Ks[buf][(krow + 32 * r) * kKS + kcol]) = kreg[r];
-    // 4x4 transpose of 16-bit values: word j of the result row for column d
-    // packs that column of two consecutive keys.
-    constexpr uint32_t LO = 0x05040100u, HI = 0x07060302u;
-    u32x2 t[4];
-    t[0] = u32x2{__builtin_amdgcn_perm(vreg[1][0], vreg[0][0], LO), __builtin_amdgcn_perm(vreg[3][0], vreg[2][0], LO)};
-    t[1] = u32x2{__builtin_amdgcn_perm(vreg[1][0], vreg[0][0], HI), __builtin_amdgcn_perm(vreg[3][0], vreg[2][0], HI)};
-    t[2] = u32x2{__builtin_amdgcn_perm(vreg[1][1], vreg[0][1], LO), __builtin_amdgcn_perm(vreg[3][1], vreg[2][1], LO)};
-    t[3] = u32x2{__builtin_amdgcn_perm(vreg[1][1], vreg[0][1], HI), __builtin_amdgcn_perm(vreg[3][1], vreg[2][1], HI)};
-#pragma unroll
-    for (int j = 0; j < 4; j++)
-      *reinterpret_cast<u32x2 *>(&Vt[buf][(vd0 + j) * kVS + vk0]) = t[j];
-  };
 
-  f32x16 accO[NQ][2];
-  float m_run[NQ], l_run[NQ];
+  // Start the ring before anything else so the first tiles overlap the Q setup.
+#pragma unroll
+  for (int t = 0; t < kStages - 1; t++)
+    if (t < nkt) issueTile(t);
+
+  // Q * c as the B operand: lane (query l32, k-slots = d 16c + 8hl .. +7).
+  v8 qf[NQ][4];
 #pragma unroll
   for (int qi = 0; qi < NQ; qi++) {
-    m_run[qi] = -INFINITY;
+    int row = q0 + qi * 32 + l32;
+    row = row < S ? row : S - 1;
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      const v8 raw = *reinterpret_cast<const v8 *>(qbase + (size_t)row * tokBytes + (16 * c + 8 * hl) * 2);
+#pragma unroll
+      for (int j = 0; j < 8; j++) qf[qi][c][j] = M::narrow(M::widen(raw[j]) * scale_log2e);
+    }
+  }
+
+  // ---- operand addresses inside a stage ---------------------------------------
+  // K: lane (key l32 [+32kb], d chunk 2c+hl) reads 16 bytes.
+  uint32_t kfrag[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++) kfrag[c] = (uint32_t)(l32 * 128 + (((2 * c + hl) ^ ((l32 >> 1) & 7)) * 16));
+  // V: as a source of the transposing read, lane L of a 16-lane group g points
+  // at key 4*hl + L/4 (+ 32kb + 16m + 8e), d = 32db + 16*(g%2) + 4*(L%4).
+  uint32_t vfrag[2];
+  {
+    const int g = lane / 16, L = lane % 16, r = L % 4, j = L / 4, jb = (j >> 1) & 1;
+#pragma unroll
+    for (int db = 0; db < 2; db++) {
+      const int chunk = (4 * db + 2 * (g % 2) + r / 2) ^ (jb << 2);
+      vfrag[db] = (uint32_t)((4 * hl + j) * 128 + chunk * 16 + 8 * (r % 2));
+    }
+  }
+
+  f32x16 accO[NQ][2];
+  f32x16 negM[NQ];       // every element: -(offset subtracted from this lane's query row)
+  float offset[NQ], l_run[NQ];
+#pragma unroll
+  for (int qi = 0; qi < NQ; qi++) {
+    offset[qi] = 0.0f;
     l_run[qi] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) negM[qi][i] = 0.0f;
 #pragma unroll
     for (int db = 0; db < 2; db++)
 #pragma unroll
       for (int i = 0; i < 16; i++) accO[qi][db][i] = 0.0f;
   }
 
-  if (nkt > 0) loadTile(0);
   for (int kt = 0; kt < nkt; kt++) {
-    const int buf = kt & 1;
-    storeTile(buf);
+    // The loads of tile kt (and of nothing later) must have landed; the barrier
+    // makes every wavefront's share visible and also says that everybody is
+    // done with tile kt-1, whose stage the next load may overwrite.
+    if (kt + 1 < nkt) asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); // vmcnt(4): tile kt+1 may still fly
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");              // vmcnt(0)
     __syncthreads();
-    if (kt + 1 < nkt) loadTile(kt + 1);
+    if (kt + kStages - 1 < nkt) issueTile(kt + kStages - 1);
 
+    const unsigned char *kst = smem + (kt % kStages) * (2 * kTileBytes);
+    const unsigned char *vst = kst + kTileBytes;
     const int key0 = kt * kBN;
+
+    // Rows of masked keys meet p = 0; zero them so that stray NaN/Inf bits in
+    // padding cannot reach the accumulators.  Only the last tile can be partial.
+    if (key0 + kBN > kvlen) {
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        const int chunk = tid + 256 * i; // 16-byte chunk of the V tile
+        if (key0 + chunk / 8 >= kvlen)
+          *reinterpret_cast<u32x4 *>(const_cast<unsigned char *>(vst) + chunk * 16) = u32x4{0u, 0u, 0u, 0u};
+      }
+      __syncthreads();
+    }
+
     // Causal: a wavefront whose queries all precede this tile has nothing to add.
     if (CAUSAL && key0 > q0 + NQ * 32 - 1) continue;
 
-    // ---- S^T = K Q^T ---------------------------------------------------
+    // ---- S^T = K (cQ)^T - m ---------------------------------------------
     f32x16 accS[NQ][2];
-#pragma unroll
-    for (int qi = 0; qi < NQ; qi++)
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) accS[qi][kb][i] = 0.0f;
 #pragma unroll
     for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
       for (int c = 0; c < 4; c++) {
-        const v8 a = *reinterpret_cast<const v8 *>(&Ks[buf][(32 * kb + l32) * kKS + 16 * c + 8 * hl]);
+        const v8 a = *reinterpret_cast<const v8 *>(kst + kb * 4096 + kfrag[c]);
 #pragma unroll
-        for (int qi = 0; qi < NQ; qi++) accS[qi][kb] = M::run(a, qf[qi][c], accS[qi][kb]);
+        for (int qi = 0; qi < NQ; qi++)
+          accS[qi][kb] = M::run(a, qf[qi][c], c == 0 ? negM[qi] : accS[qi][kb]);
       }
     }
 
@@ -248,31 +343,40 @@ __global__ __launch_bounds__(256) void fmha_fwd_d64_kernel(const uint16_t *__res
       for (int kb = 0; kb < 2; kb++)
 #pragma unroll
         for (int i = 0; i < 16; i++) mx = fmaxf(mx, accS[qi][kb][i]);
-      mx = halves_max(mx);
-      const float m_new = fmaxf(m_run[qi], mx);
-      const float alpha = __builtin_amdgcn_exp2f((m_run[qi] - m_new) * scale_log2e);
-      const float mc = m_new * scale_log2e;
-      float lsum = 0.0f;
+      mx = halves_max(mx); // row maximum relative to the current offset
+      // Re-centre when some row of the wavefront needs it; the first tile
+      // always does (its offset is the placeholder 0 and O, l are still zero).
+      if (kt == 0 || __builtin_amdgcn_ballot_w64(mx > kLazyLog2) != 0) {
+        const float delta = kt == 0 ? mx : fmaxf(mx, 0.0f);
+        offset[qi] += delta;
 #pragma unroll
-      for (int kb = 0; kb < 2; kb++)
+        for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-          const float p = __builtin_amdgcn_exp2f(accS[qi][kb][i] * scale_log2e - mc);
-          accS[qi][kb][i] = p;
-          lsum += p;
+          for (int i = 0; i < 16; i++) accS[qi][kb][i] -= delta;
+        if (kt != 0) {
+          const float alpha = __builtin_amdgcn_exp2f(-delta);
+          l_run[qi] *= alpha;
+#pragma unroll
+          for (int db = 0; db < 2; db++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) accO[qi][db][i] *= alpha;
         }
-      l_run[qi] = l_run[qi] * alpha + lsum;
-      m_run[qi] = m_new;
+        const float nm = -offset[qi];
 #pragma unroll
-      for (int db = 0; db < 2; db++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) accO[qi][db][i] *= alpha;
+        for (int i = 0; i < 16; i++) negM[qi][i] = nm;
+      }
+      float lsum = l_run[qi];
 #pragma unroll
       for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-        for (int m = 0; m < 2; m++)
+        for (int m = 0; m < 2; m++) {
 #pragma unroll
-          for (int j = 0; j < 8; j++) pf[qi][kb][m][j] = M::narrow(accS[qi][kb][8 * m + j]);
+          for (int j = 0; j < 8; j++)
+            pf[qi][kb][m][j] = M::narrow(__builtin_amdgcn_exp2f(accS[qi][kb][8 * m + j]));
+#pragma unroll
+          for (int w = 0; w < 4; w++) lsum = M::pairSum(pf[qi][kb][m], w, lsum);
+        }
+      l_run[qi] = lsum;
     }
 
     // ---- O^T += V^T P^T ----------------------------------------------------
@@ -282,9 +386,9 @@ __global__ __launch_bounds__(256) void fmha_fwd_d64_kernel(const uint16_t *__res
       for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
         for (int m = 0; m < 2; m++) {
-          const uint16_t *vrow = &Vt[buf][(32 * db + l32) * kVS + 32 * kb + 16 * m + 4 * hl];
-          const v4 lo = *reinterpret_cast<const v4 *>(vrow);
-          const v4 hi = *reinterpret_cast<const v4 *>(vrow + 8);
+          const unsigned char *vp = vst + vfrag[db] + (32 * kb + 16 * m) * 128;
+          const v4 lo = M::readTr(vp);            // k-slots 0..3: keys +4hl+0..3
+          const v4 hi = M::readTr(vp + 8 * 128);  // k-slots 4..7: keys +8+4hl+0..3
           const v8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
           for (int qi = 0; qi < NQ; qi++) accO[qi][db] = M::run(a, pf[qi][kb][m], accO[qi][db]);
@@ -293,23 +397,38 @@ __global__ __launch_bounds__(256) void fmha_fwd_d64_kernel(const uint16_t *__res
     }
   }
 
-  // ---- normalise and store -------------------------------------------------
+  // ---- normalise, transpose through LDS, store whole rows ------------------
+  __syncthreads(); // every wavefront is done reading the K / V tiles
+  uint16_t *stage = reinterpret_cast<uint16_t *>(smem) + wave * (NQ * 32 * kOS);
+  static_assert(4 * NQ * 32 * kOS * 2 <= kStages * 2 * kTileBytes, "output staging must fit in the ring");
 #pragma unroll
   for (int qi = 0; qi < NQ; qi++) {
     const float l = halves_sum(l_run[qi]);
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    const int query = q0 + qi * 32 + l32;
+#pragma unroll
+    for (int db = 0; db < 2; db++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        v4 o;
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = M::narrow(accO[qi][db][4 * g + i] * inv);
+        *reinterpret_cast<v4 *>(&stage[(qi * 32 + l32) * kOS + 32 * db + 8 * g + 4 * hl]) = o;
+      }
+  }
+  // Each wavefront reads back only what it wrote: no block barrier needed, the
+  // LDS accesses of one wavefront are ordered.
+#pragma unroll
+  for (int it = 0; it < NQ * 4; it++) {
+    const int chunk = it * 64 + lane; // 16-byte chunk index inside the wave's tile
+    const int r = chunk / 8, cidx = chunk % 8;
+    const int query = q0 + r;
     if (query < S) {
-      uint16_t *orow = out + ((size_t)b * S + query) * H * kD + (size_t)h * kD;
-#pragma unroll
-      for (int db = 0; db < 2; db++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          v4 o;
-#pragma unroll
-          for (int i = 0; i < 4; i++) o[i] = M::narrow(accO[qi][db][4 * g + i] * inv);
-          *reinterpret_cast<v4 *>(orow + 32 * db + 8 * g + 4 * hl) = o;
-        }
+      // 8-byte LDS reads: the staging stride is 8-byte but not 16-byte aligned
+      const u32x2 lo = *reinterpret_cast<const u32x2 *>(&stage[r * kOS + cidx * 8]);
+      const u32x2 hi = *reinterpret_cast<const u32x2 *>(&stage[r * kOS + cidx * 8 + 4]);
+      const u32x4 val = {lo[0], lo[1], hi[0], hi[1]};
+      __builtin_nontemporal_store(
+          val, reinterpret_cast<u32x4 *>(out + ((size_t)b * S + query) * H * kD + (size_t)h * kD + cidx * 8));
     }
   }
 }
@@ -341,12 +460,14 @@ void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int 
   if (!qkv || !out) fail("fusedMHA: null pointer");
   if (!aligned16(qkv) || !aligned16(out)) fail("fusedMHA: qkv and out must be 16-byte aligned");
   if (!(scale > 0.0f) || !(scale < INFINITY)) fail("fusedMHA: softmax scale must be positive and finite");
-  if (dt == DType::F16)
+  if ((int64_t)S * 3 * H * kD * 2 > 0x7fffffffLL) fail("fusedMHA: one sequence of QKV must stay below 2 GiB");
+  if (dt == DType::F16) {
     launch<_Float16, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
-  else if (dt == DType::BF16)
+  } else if (dt == DType::BF16) {
     launch<bf16_t, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
-  else
+  } else {
     fail("fusedMHA: element type must be fp16 or bf16");
+  }
 }
 
 } // namespace mgpu

@@ -6,7 +6,8 @@
 // a row lives in the registers of one group of 16/32/64 lanes:
 //   one 128-bit coalesced load per vector, statistics in fp32 with a two-pass
 //   (mean, then centred sum of squares) reduction over registers and DPP /
-//   lane-exchange sums, one 128-bit store per vector.  One pass over HBM.
+//   lane-exchange sums, one 128-bit non-temporal store per vector (plain loads
+//   + non-temporal stores measured fastest on MI355X).  One pass over HBM.
 // Rows wider than a wavefront can hold, rows whose length is not a multiple of
 // the vector width, and unaligned pointers take a block-per-row kernel.
 #include "common.hpp"
@@ -46,8 +47,8 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
     for (int k = 0; k < VPL; k++) {
       const int v = lane + k * LANES;
       if (v < nvec) {
-        raw[k] = __builtin_nontemporal_load(xv + v);
-        if (RESIDUAL) rawr[k] = __builtin_nontemporal_load(rv + v);
+        raw[k] = xv[v];
+        if (RESIDUAL) rawr[k] = rv[v];
       }
     }
 

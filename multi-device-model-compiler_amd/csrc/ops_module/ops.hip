@@ -26,7 +26,6 @@ extern "C" __global__ __launch_bounds__(256) void main_graph_kernel(const float 
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   for (int64_t i = tid; i < n4; i += stride)
-    __builtin_nontemporal_store(__builtin_nontemporal_load(a4 + i) + __builtin_nontemporal_load(b4 + i),
-                                c4 + i);
+    __builtin_nontemporal_store(a4[i] + b4[i], c4 + i);
   for (int64_t i = n4 * 4 + tid; i < n; i += stride) c[i] = a[i] + b[i];
 }
