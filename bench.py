@@ -36,6 +36,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 MALL_BYTES = 256 << 20
+# HBM bytes per launch of the headline kernel, from two rocprofv3 --pmc passes
+# (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0, the factors a 64 MiB device copy
+# gives for the same counters); see profiles/layernorm_f32_hbm_traffic.md.
+LN_F32_TRAFFIC_BYTES = 25_240_000
 
 
 def parse_args():
@@ -46,6 +50,8 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="enqueue launches directly instead of through a hipGraph")
     ap.add_argument("--only", type=str, default="", help="comma list of kernels to run besides the headline")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run plain device copies of 64 MiB (for scaling FETCH_SIZE / WRITE_SIZE counters)")
     return ap.parse_args()
 
 
@@ -145,6 +151,16 @@ def main():
     gen.manual_seed(20241)
     kernels = []
 
+    if args.copy_calibration:
+        # A copy of known size: 64 MiB read + 64 MiB written per launch.  The
+        # FETCH_SIZE / WRITE_SIZE a profiler reports for it give the factor by
+        # which the same counters of the other kernels are scaled.
+        src = torch.empty(64 << 20, dtype=torch.uint8, device=dev).random_(generator=gen)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+
     # ---------------- headline: LayerNorm fp32 (32,128,768) -------------------
     m, n = 32 * 128, 768
     ln_bytes = 2 * m * n * 4 + 2 * n * 4
@@ -165,6 +181,7 @@ def main():
     check()
     headline = hbm_entry("layernorm_f32", "LayerNorm fp32 (32,128,768) eps=1e-5 [configs[1]]", "f32",
                          ln_bytes, ms_cold, K, ms_warm)
+    headline["roofline"]["traffic"] = LN_F32_TRAFFIC_BYTES
     del xs, ys
 
     # ---------------- LayerNorm fp16 ------------------------------------------
