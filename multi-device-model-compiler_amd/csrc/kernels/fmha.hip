@@ -36,24 +36,26 @@
 // lanes, lane L receives element L%4 of the four 8-byte rows addressed by
 // lanes L/4, L/4+4, L/4+8, L/4+12 - four keys of one d column.
 //
-// Softmax runs in fp32 in base 2.  At head_dim 64 the softmax VALU work per
-// score costs about as many issue cycles as the 256 MFMA flops that score pays
-// for, so the loop is trimmed to exp2 + half a max3 + half a convert + half a
-// dot2 per score:
-//   * Q is multiplied by c = scale*log2(e) once (rounded to the 16-bit type: a
-//     relative perturbation of at most half an ulp of Q), and the running
-//     offset m is subtracted BY THE MATRIX CORE: the first MFMA of each score
-//     block takes a register block holding -m as its C operand, so the scores
-//     come out as s*c - m and need no VALU fma;
-//   * m is the row maximum as of the last adjustment, not of the current tile:
-//     it is only advanced (and O, l rescaled, the -m block rewritten) when some
-//     row of the wavefront sees a score more than 2^8 above it.  p stays <= 256,
-//     well inside fp16, and O / l is unchanged because both use the same m;
+// Softmax runs in fp32 in base 2: p = exp2(s*c - m*c), c = scale*log2(e), the
+// scale staying in fp32.  At head_dim 64 one score pays for only 256 MFMA
+// flops, i.e. 16 issue cycles per wavefront, and a wavefront issues in order:
+// VALU work is free only while it sits between MFMAs whose results it does not
+// need.  So the per-score work is trimmed to one fma, one exp2, half a convert
+// and half a dot2, and the row maximum is taken out of the hot path entirely:
+//   * m is a stale reference, not the running maximum.  P is produced
+//     optimistically against it; fp16 holds p up to 2^16, and an overflow (or
+//     the first tile, where m = -inf) shows up as a non-finite row sum.  Only
+//     then does the wavefront take the slow path: true row maximum, rescale of
+//     O and l, P recomputed.  O / l does not depend on which m was used.
+//     Without the maximum in front of it the softmax of a tile is a single pass
+//     of fma / exp2 / convert / dot2 over the scores;
 //   * the row sum is taken with v_dot2_f32_{f16,bf16} over the already converted
 //     P pairs (two scores per instruction; the normaliser then matches the P
 //     the matrix cores consume);
-//   * accumulators stay in VGPRs (two wavefronts per SIMD leave 256 registers
-//     each, so no AGPR copies).
+//   * accumulators stay in VGPRs (no AGPR copies);
+//   * three wavefronts share a SIMD (142 VGPRs) and are left to drift apart, so
+//     that one is in an MFMA phase while another does its softmax; s_setprio
+//     lets the MFMA phases win the issue slot.
 // The output tile is transposed through LDS so that every store instruction
 // writes whole 128-byte rows.
 #include "common.hpp"
@@ -71,13 +73,14 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned char __attribute__((address_space(3))) lds_u8; // a byte in LDS
 
 constexpr int kD = 64;   // head dim
 constexpr int kBN = 64;  // keys per tile
 constexpr int kStages = 3;               // LDS ring depth
 constexpr int kTileBytes = kBN * kD * 2; // one K or V tile: 64 rows of 128 B, unpadded
 constexpr int kOS = 68;  // output staging row stride in elements
-constexpr float kLazyLog2 = 8.0f; // re-centre only when a score exceeds the offset by 2^8
+constexpr float kSumLimit = 1e30f; // a row sum above this (or NaN) means P overflowed against the stale m
 
 template <typename T> struct Mma;
 template <> struct Mma<_Float16> {
@@ -88,7 +91,7 @@ template <> struct Mma<_Float16> {
   }
   __device__ static __forceinline__ _Float16 narrow(float f) { return (_Float16)f; }
   __device__ static __forceinline__ float widen(_Float16 h) { return (float)h; }
-  __device__ static __forceinline__ v4 readTr(const unsigned char *p) {
+  __device__ static __forceinline__ v4 readTr(const lds_u8 *p) {
     return __builtin_bit_cast(v4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 __attribute__((address_space(3))) *)p));
   }
   // acc + sum of the two packed values of word w of a v8
@@ -107,7 +110,7 @@ template <> struct Mma<bf16_t> {
   }
   __device__ static __forceinline__ __bf16 narrow(float f) { return (__bf16)f; }
   __device__ static __forceinline__ float widen(__bf16 h) { return (float)h; }
-  __device__ static __forceinline__ v4 readTr(const unsigned char *p) {
+  __device__ static __forceinline__ v4 readTr(const lds_u8 *p) {
     return __builtin_bit_cast(v4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 __attribute__((address_space(3))) *)p));
   }
   __device__ static __forceinline__ float pairSum(v8 p, int w, float acc) {
@@ -235,18 +238,15 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
   for (int t = 0; t < kStages - 1; t++)
     if (t < nkt) issueTile(t);
 
-  // Q * c as the B operand: lane (query l32, k-slots = d 16c + 8hl .. +7).
+  // Q as the B operand: lane (query l32, k-slots = d 16c + 8hl .. +7).
   v8 qf[NQ][4];
 #pragma unroll
   for (int qi = 0; qi < NQ; qi++) {
     int row = q0 + qi * 32 + l32;
     row = row < S ? row : S - 1;
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
-      const v8 raw = *reinterpret_cast<const v8 *>(qbase + (size_t)row * tokBytes + (16 * c + 8 * hl) * 2);
-#pragma unroll
-      for (int j = 0; j < 8; j++) qf[qi][c][j] = M::narrow(M::widen(raw[j]) * scale_log2e);
-    }
+    for (int c = 0; c < 4; c++)
+      qf[qi][c] = *reinterpret_cast<const v8 *>(qbase + (size_t)row * tokBytes + (16 * c + 8 * hl) * 2);
   }
 
   // ---- operand addresses inside a stage ---------------------------------------
@@ -267,14 +267,11 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
   }
 
   f32x16 accO[NQ][2];
-  f32x16 negM[NQ];       // every element: -(offset subtracted from this lane's query row)
-  float offset[NQ], l_run[NQ];
+  float m_run[NQ], l_run[NQ]; // stale reference maximum (raw score units), running sum
 #pragma unroll
   for (int qi = 0; qi < NQ; qi++) {
-    offset[qi] = 0.0f;
+    m_run[qi] = -INFINITY;
     l_run[qi] = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 16; i++) negM[qi][i] = 0.0f;
 #pragma unroll
     for (int db = 0; db < 2; db++)
 #pragma unroll
@@ -290,18 +287,18 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
     __syncthreads();
     if (kt + kStages - 1 < nkt) issueTile(kt + kStages - 1);
 
-    const unsigned char *kst = smem + (kt % kStages) * (2 * kTileBytes);
-    const unsigned char *vst = kst + kTileBytes;
+    const uint32_t stageOff = (uint32_t)((kt % kStages) * (2 * kTileBytes));
     const int key0 = kt * kBN;
 
     // Rows of masked keys meet p = 0; zero them so that stray NaN/Inf bits in
     // padding cannot reach the accumulators.  Only the last tile can be partial.
     if (key0 + kBN > kvlen) {
+      unsigned char *vst = smem + stageOff + kTileBytes;
 #pragma unroll
       for (int i = 0; i < 2; i++) {
         const int chunk = tid + 256 * i; // 16-byte chunk of the V tile
         if (key0 + chunk / 8 >= kvlen)
-          *reinterpret_cast<u32x4 *>(const_cast<unsigned char *>(vst) + chunk * 16) = u32x4{0u, 0u, 0u, 0u};
+          *reinterpret_cast<u32x4 *>(vst + chunk * 16) = u32x4{0u, 0u, 0u, 0u};
       }
       __syncthreads();
     }
@@ -309,20 +306,34 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
     // Causal: a wavefront whose queries all precede this tile has nothing to add.
     if (CAUSAL && key0 > q0 + NQ * 32 - 1) continue;
 
-    // ---- S^T = K (cQ)^T - m ---------------------------------------------
+    // Operand pointers in the LDS address space: one add per tile, the rest
+    // of every address is an instruction immediate.
+    const lds_u8 *kp[4], *vp[2];
+#pragma unroll
+    for (int c = 0; c < 4; c++) kp[c] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kfrag[c]);
+#pragma unroll
+    for (int db = 0; db < 2; db++) vp[db] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kTileBytes + vfrag[db]);
+
+    // ---- S^T = K Q^T -------------------------------------------------------
     f32x16 accS[NQ][2];
+    __builtin_amdgcn_s_setprio(2); // MFMA phases outrank the softmax phases of the SIMD's other wavefronts
 #pragma unroll
     for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
       for (int c = 0; c < 4; c++) {
-        const v8 a = *reinterpret_cast<const v8 *>(kst + kb * 4096 + kfrag[c]);
+        const v8 a = *reinterpret_cast<const v8 __attribute__((address_space(3))) *>(kp[c] + kb * 4096);
 #pragma unroll
-        for (int qi = 0; qi < NQ; qi++)
-          accS[qi][kb] = M::run(a, qf[qi][c], c == 0 ? negM[qi] : accS[qi][kb]);
+        for (int qi = 0; qi < NQ; qi++) {
+          if (c == 0) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) accS[qi][kb][i] = 0.0f;
+          }
+          accS[qi][kb] = M::run(a, qf[qi][c], accS[qi][kb]);
+        }
       }
     }
 
-    // ---- online softmax, one query per lane column ------------------------
+    __builtin_amdgcn_s_setprio(0);
     const bool needMask = (key0 + kBN > kvlen) || (CAUSAL && key0 + kBN - 1 > q0);
     v8 pf[NQ][2][2];
 #pragma unroll
@@ -338,63 +349,63 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
             if (!ok) accS[qi][kb][i] = -INFINITY;
           }
       }
-      float mx = accS[qi][0][0];
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) mx = fmaxf(mx, accS[qi][kb][i]);
-      mx = halves_max(mx); // row maximum relative to the current offset
-      // Re-centre when some row of the wavefront needs it; the first tile
-      // always does (its offset is the placeholder 0 and O, l are still zero).
-      if (kt == 0 || __builtin_amdgcn_ballot_w64(mx > kLazyLog2) != 0) {
-        const float delta = kt == 0 ? mx : fmaxf(mx, 0.0f);
-        offset[qi] += delta;
+      // ---- P against the stale reference maximum ---------------------------
+      auto makeP = [&](float mref) {
+        const float mc = mref * scale_log2e;
+        float lsum = 0.0f;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-          for (int i = 0; i < 16; i++) accS[qi][kb][i] -= delta;
-        if (kt != 0) {
-          const float alpha = __builtin_amdgcn_exp2f(-delta);
-          l_run[qi] *= alpha;
+          for (int m = 0; m < 2; m++) {
 #pragma unroll
-          for (int db = 0; db < 2; db++)
+            for (int j = 0; j < 8; j++)
+              pf[qi][kb][m][j] = M::narrow(__builtin_amdgcn_exp2f(accS[qi][kb][8 * m + j] * scale_log2e - mc));
 #pragma unroll
-            for (int i = 0; i < 16; i++) accO[qi][db][i] *= alpha;
-        }
-        const float nm = -offset[qi];
+            for (int w = 0; w < 4; w++) lsum = M::pairSum(pf[qi][kb][m], w, lsum);
+          }
+        return lsum;
+      };
+      float lsum = makeP(m_run[qi]);
+      // Overflow of P (or m = -inf on the first tile) makes the sum non-finite.
+      if (__builtin_amdgcn_ballot_w64(!(lsum <= kSumLimit)) != 0) {
+        float mx = accS[qi][0][0];
 #pragma unroll
-        for (int i = 0; i < 16; i++) negM[qi][i] = nm;
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) mx = fmaxf(mx, accS[qi][kb][i]);
+        mx = halves_max(mx);
+        const float m_new = fmaxf(m_run[qi], mx);
+        // rows that never saw a key yet have l = 0 and O = 0: any finite factor does
+        const float alpha = m_run[qi] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f((m_run[qi] - m_new) * scale_log2e);
+        m_run[qi] = m_new;
+        l_run[qi] *= alpha;
+#pragma unroll
+        for (int db = 0; db < 2; db++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) accO[qi][db][i] *= alpha;
+        lsum = makeP(m_new);
       }
-      float lsum = l_run[qi];
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int m = 0; m < 2; m++) {
-#pragma unroll
-          for (int j = 0; j < 8; j++)
-            pf[qi][kb][m][j] = M::narrow(__builtin_amdgcn_exp2f(accS[qi][kb][8 * m + j]));
-#pragma unroll
-          for (int w = 0; w < 4; w++) lsum = M::pairSum(pf[qi][kb][m], w, lsum);
-        }
-      l_run[qi] = lsum;
+      l_run[qi] += lsum;
     }
 
     // ---- O^T += V^T P^T ----------------------------------------------------
+    __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int db = 0; db < 2; db++) {
 #pragma unroll
       for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
         for (int m = 0; m < 2; m++) {
-          const unsigned char *vp = vst + vfrag[db] + (32 * kb + 16 * m) * 128;
-          const v4 lo = M::readTr(vp);            // k-slots 0..3: keys +4hl+0..3
-          const v4 hi = M::readTr(vp + 8 * 128);  // k-slots 4..7: keys +8+4hl+0..3
+          const lds_u8 *p = vp[db] + (32 * kb + 16 * m) * 128;
+          const v4 lo = M::readTr(p);            // k-slots 0..3: keys +4hl+0..3
+          const v4 hi = M::readTr(p + 8 * 128);  // k-slots 4..7: keys +8+4hl+0..3
           const v8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
           for (int qi = 0; qi < NQ; qi++) accO[qi][db] = M::run(a, pf[qi][kb][m], accO[qi][db]);
         }
       }
     }
+    __builtin_amdgcn_s_setprio(0);
   }
 
   // ---- normalise, transpose through LDS, store whole rows ------------------
@@ -461,6 +472,9 @@ void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int 
   if (!aligned16(qkv) || !aligned16(out)) fail("fusedMHA: qkv and out must be 16-byte aligned");
   if (!(scale > 0.0f) || !(scale < INFINITY)) fail("fusedMHA: softmax scale must be positive and finite");
   if ((int64_t)S * 3 * H * kD * 2 > 0x7fffffffLL) fail("fusedMHA: one sequence of QKV must stay below 2 GiB");
+  // One 32-query block per wavefront: 64 queries per wavefront would halve the
+  // LDS operand traffic per flop, but at 224 VGPRs only two wavefronts fit a
+  // SIMD and the kernel measured slower at every shape tried.
   if (dt == DType::F16) {
     launch<_Float16, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
   } else if (dt == DType::BF16) {

@@ -1,6 +1,9 @@
 """Parity of the HIP fused multi-head attention (C ABI mgpuFusedMHAF16 / BF16)
-with the oracle: max absolute error <= 2e-3 on fp16 outputs against the fp32/64
-CPU result (bf16: <= 8e-3, its output spacing below 1 being 2^-8)."""
+with the oracle, on unit-variance inputs (logits ~ N(0, 1) at scale 1/8, outputs
+O(0.1 .. 1)): |error| <= 2e-3 * max(1, |ref|) elementwise on fp16 outputs
+against the fp64 CPU result, i.e. max abs error <= 2e-3 wherever the output is
+below 1 and one fp16 spacing above that (bf16: 8e-3, its spacing below 1 being
+2^-8)."""
 import numpy as np
 import pytest
 
@@ -12,12 +15,19 @@ TOL_F16 = 2e-3
 TOL_BF16 = 8e-3
 
 
+def excess(got, ref, tol):
+    """Largest |got - ref| in units of the allowed bound tol * max(1, |ref|)."""
+    return float((np.abs(got - ref) / (tol * np.maximum(1.0, np.abs(ref)))).max()) if ref.size else 0.0
+
+
 def run(pkg, gpu, qkv, lens=None, causal=False, scale=None):
     tl = to_dev(np.asarray(lens, np.int32), gpu) if lens is not None else None
     return pkg.fused_mha(to_dev(qkv, gpu), tl, scale=scale, causal=causal).cpu().numpy().astype(np.float32)
 
 
-def make_qkv(rng, B, S, H, std=1.0 / 8):
+def make_qkv(rng, B, S, H, std=1.0):
+    # unit variance: logits ~ N(0, 1) at scale 1/8, outputs O(0.1 .. 1) - an error in
+    # the softmax weights or a V tile paired with the wrong P is far above tolerance
     return (rng.standard_normal((B, S, 3, H, 64)) * std).astype(np.float16)
 
 
@@ -25,7 +35,7 @@ def test_fmha_config2_b32_s128_h12(pkg, gpu, oracle):
     rng = np.random.Generator(np.random.PCG64(20242))
     qkv = make_qkv(rng, 32, 128, 12)
     got = run(pkg, gpu, qkv)
-    assert np.abs(got - oracle.fmha(qkv)).max() <= TOL_F16
+    assert excess(got, oracle.fmha(qkv), TOL_F16) <= 1.0
 
 
 def test_fmha_config3_b8_s512_h16_key_padding(pkg, gpu, oracle):
@@ -33,14 +43,14 @@ def test_fmha_config3_b8_s512_h16_key_padding(pkg, gpu, oracle):
     qkv = make_qkv(rng, 8, 512, 16)
     lens = rng.integers(256, 513, 8).astype(np.int32)
     got = run(pkg, gpu, qkv, lens)
-    assert np.abs(got - oracle.fmha(qkv, lens)).max() <= TOL_F16
+    assert excess(got, oracle.fmha(qkv, lens), TOL_F16) <= 1.0
 
 
 def test_fmha_roofline_shape_b32_s512_h12(pkg, gpu, oracle):
     rng = np.random.Generator(np.random.PCG64(20244))
     qkv = make_qkv(rng, 32, 512, 12)
     got = run(pkg, gpu, qkv)
-    assert np.abs(got - oracle.fmha(qkv)).max() <= TOL_F16
+    assert excess(got, oracle.fmha(qkv), TOL_F16) <= 1.0
 
 
 # ragged S (partial query blocks and partial key tiles), S below one tile,
@@ -54,7 +64,7 @@ def test_fmha_ragged_and_masked(pkg, gpu, oracle, rng, B, S, H, lens):
     qkv = make_qkv(rng, B, S, H)
     got = run(pkg, gpu, qkv, lens)
     ref = oracle.fmha(qkv, lens)
-    assert np.abs(got - ref).max() <= TOL_F16
+    assert excess(got, ref, TOL_F16) <= 1.0
     if lens is not None:
         for b, l in enumerate(lens):
             if l <= 0:
@@ -66,27 +76,26 @@ def test_fmha_ragged_and_masked(pkg, gpu, oracle, rng, B, S, H, lens):
 def test_fmha_causal(pkg, gpu, oracle, rng, B, S, H, lens):
     qkv = make_qkv(rng, B, S, H)
     got = run(pkg, gpu, qkv, lens, causal=True)
-    assert np.abs(got - oracle.fmha(qkv, lens, causal=True)).max() <= TOL_F16
+    assert excess(got, oracle.fmha(qkv, lens, causal=True), TOL_F16) <= 1.0
 
 
 def test_fmha_large_logits_and_other_scales(pkg, gpu, oracle, rng):
-    """Peaked softmax rows exercise the lazy re-centring of the running offset;
-    the scale is a free parameter of the entry point.
-
-    The kernel folds scale*log2(e) into Q once, rounded to fp16: every logit is
-    perturbed by at most 2^-11 relative per Q element.  With unit-variance q, k
-    and scale 0.125 (logits ~ N(0,1)) that stays far inside 2e-3; at scale 1.0
-    the logits reach |40| in log2 units, softmax weights move by up to ~1 % and
-    the bound below is the documented one for that regime."""
-    qkv = make_qkv(rng, 2, 256, 2, std=1.0)
-    for scale, tol in ((0.125, TOL_F16), (0.01, TOL_F16), (1.0, 2e-2)):
+    """Peaked softmax rows: the kernel produces P against a stale reference
+    maximum and repairs overflow after the fact, so rows whose scores keep
+    growing from tile to tile (scale 1.0: logits ~ N(0, 64), up to +-40) take
+    the repair path over and over.  The scale is a free fp32 parameter of the
+    entry point and is applied in fp32, so the bound does not move with it."""
+    qkv = make_qkv(rng, 2, 256, 2)
+    for scale in (0.01, 0.125, 0.5, 1.0):
         got = run(pkg, gpu, qkv, scale=scale)
-        err = np.abs(got - oracle.fmha(qkv, scale=scale)).max()
-        assert err <= tol, (scale, err)
-    # moderately peaked rows at the benchmark scale: |logits| up to ~12
-    qkv = make_qkv(rng, 2, 320, 2, std=1.6)
-    err = np.abs(run(pkg, gpu, qkv) - oracle.fmha(qkv)).max()
-    assert err <= 4e-3, err
+        assert excess(got, oracle.fmha(qkv, scale=scale), TOL_F16) <= 1.0, scale
+    for std in (1.6, 3.0):  # |logits| up to ~12 and ~40 at the default scale, outputs up to ~13
+        qkv = make_qkv(rng, 2, 320, 2, std=std)
+        assert excess(run(pkg, gpu, qkv), oracle.fmha(qkv), TOL_F16) <= 1.0, std
+    # a row maximum that rises by far more than fp16's range from one tile to the next
+    qkv = make_qkv(rng, 1, 256, 1)
+    qkv[0, :, 1, 0, :] *= np.linspace(0.05, 6.0, 256, dtype=np.float16)[:, None]
+    assert excess(run(pkg, gpu, qkv, scale=1.0), oracle.fmha(qkv, scale=1.0), TOL_F16) <= 1.0
 
 
 def test_fmha_padding_garbage_is_ignored(pkg, gpu, oracle, rng):
@@ -99,7 +108,7 @@ def test_fmha_padding_garbage_is_ignored(pkg, gpu, oracle, rng):
         dirty[b, l:, 1:] = np.float16(np.nan)
         dirty[b, l::2, 1:] = np.float16(np.inf)
     got = run(pkg, gpu, dirty, lens)
-    assert np.isfinite(got).all() and np.abs(got - ref).max() <= TOL_F16
+    assert np.isfinite(got).all() and excess(got, ref, TOL_F16) <= 1.0
 
 
 def test_fmha_identities_at_full_size(pkg, gpu):
@@ -110,7 +119,7 @@ def test_fmha_identities_at_full_size(pkg, gpu):
     g = torch.Generator(device=gpu)
     g.manual_seed(11)
     B, S, H = 32, 512, 12
-    qkv = (torch.randn((B, S, 3, H, 64), device=gpu, generator=g) / 8).half()
+    qkv = torch.randn((B, S, 3, H, 64), device=gpu, generator=g).half()
     base = pkg.fused_mha(qkv).float()
     c = qkv.clone()
     c[:, :, 2] = 0.375
@@ -122,17 +131,17 @@ def test_fmha_identities_at_full_size(pkg, gpu):
     perm = torch.randperm(S, device=gpu, generator=g)
     p = qkv.clone()
     p[:, :, 1:] = qkv[:, perm, 1:]
-    assert (pkg.fused_mha(p).float() - base).abs().max().item() <= 1e-3
+    assert (pkg.fused_mha(p).float() - base).abs().max().item() <= 2e-3
     assert torch.equal(pkg.fused_mha(qkv), pkg.fused_mha(qkv))  # deterministic
 
 
 def test_fmha_bf16(pkg, gpu, oracle, rng):
     import torch
     for (B, S, H, lens, causal) in [(2, 128, 2, None, False), (2, 200, 3, [200, 77], False), (1, 130, 1, None, True)]:
-        f = (rng.standard_normal((B, S, 3, H, 64)) / 8).astype(np.float32)
+        f = rng.standard_normal((B, S, 3, H, 64)).astype(np.float32)
         t = torch.from_numpy(f).to(gpu).to(torch.bfloat16)
         tl = to_dev(np.asarray(lens, np.int32), gpu) if lens is not None else None
         got = pkg.fused_mha(t, tl, causal=causal).float().cpu().numpy()
         bits = t.view(torch.int16).cpu().numpy().view(np.uint16)
         ref = oracle.fmha(bits, lens, causal=causal, bf16=True)
-        assert np.abs(got - ref).max() <= TOL_BF16
+        assert excess(got, ref, TOL_BF16) <= 1.0
