@@ -5,10 +5,15 @@
 // Same flags, call order and output lines as the reference's
 // tools/multi-device-gpu-runner/multi-device-gpu-runner.cpp:19-93; the
 // differences are the argument parser (no LLVM), `--ops` defaulting to
-// ./ops.hsaco (a gfx950 code object instead of ops.cubin) and `--dtype`.
+// ./ops.hsaco (a gfx950 code object instead of ops.cubin) and `--dtype`.  A
+// `<name>.plan` in place of the library runs that device plan through its GPU
+// lowering; shapes and element types then come from the plan and --input /
+// --output / --dtype are ignored.
+#include "mgpu_ops.h"
 #include "multi-device-model-compiler/Kernels/GPU/Ops.h"
 #include "multi-device-model-compiler/Runtime/HIP/HipRuntimeWrappers.h"
 #include "multi-device-model-compiler/Runtime/ModelInfo.h"
+#include "multi-device-model-compiler/Runtime/PlanModel.h"
 #include "multi-device-model-compiler/Runtime/RuntimeUtil.h"
 #include "multi-device-model-compiler/Runtime/TensorDescripter.h"
 
@@ -33,6 +38,39 @@ int main(int argc, char **argv) {
 
   mgpuModuleFileLoad(OpsLibPath.str().c_str());
   gpuOpsInit();
+
+  if (IsPlanFile(LibPath.str())) {
+    PlanModel *model = PlanModel::Load(LibPath.str(), conversion::DeviceType::GPU);
+    if (!model || !model->PrepareIO(InputData.values) || !model->Run())
+      return 1;
+    if (!OutputName.str().empty())
+      model->SaveOutput(0, OutputName.str());
+    const int reruns = RerunTimes.asInt();
+    if (reruns != 0) {
+      auto stream = mgpuStreamCreate();
+      auto eventBegin = mgpuEventEnableTimeCreate(), eventEnd = mgpuEventEnableTimeCreate();
+      float elapsed = 0;
+      for (int i = 0; i < reruns; ++i) {
+        mgpuEventRecord(eventBegin, stream);
+        if (!model->Run())
+          return 1;
+        mgpuEventRecord(eventEnd, stream);
+        mgpuEventSynchronize(eventEnd);
+        elapsed += mgpuEventElapsedTime(eventBegin, eventEnd);
+      }
+      mgpuEventDestroy(eventBegin);
+      mgpuEventDestroy(eventEnd);
+      mgpuStreamDestroy(stream);
+      std::printf("Run \t%d\ttimes\n", reruns);
+      std::printf("Average time:\t%g\tseconds\n", elapsed / (reruns * 1000.0f));
+    }
+    if (const char *err = mgpuOpsTakeLastError())
+      std::fprintf(stderr, "%s\n", err);
+    delete model;
+    gpuOpsDeinit();
+    mgpuModuleUnload();
+    return 0;
+  }
 
   ModelInfo *info = ModelInfo::ParseModelInfo();
   if (!info)

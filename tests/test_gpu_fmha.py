@@ -33,6 +33,9 @@ def make_qkv(rng, B, S, H, std=1.0):
 
 def test_fmha_config2_b32_s128_h12(pkg, gpu, oracle):
     rng = np.random.Generator(np.random.PCG64(20242))
+    qkv = make_qkv(rng, 32, 128, 12, std=1.0 / 8)  # the configuration's own draw
+    got = run(pkg, gpu, qkv)
+    assert np.abs(got - oracle.fmha(qkv)).max() <= TOL_F16
     qkv = make_qkv(rng, 32, 128, 12)
     got = run(pkg, gpu, qkv)
     assert excess(got, oracle.fmha(qkv), TOL_F16) <= 1.0
@@ -40,8 +43,11 @@ def test_fmha_config2_b32_s128_h12(pkg, gpu, oracle):
 
 def test_fmha_config3_b8_s512_h16_key_padding(pkg, gpu, oracle):
     rng = np.random.Generator(np.random.PCG64(20243))
-    qkv = make_qkv(rng, 8, 512, 16)
     lens = rng.integers(256, 513, 8).astype(np.int32)
+    qkv = make_qkv(rng, 8, 512, 16, std=1.0 / 8)  # the configuration's own draw
+    got = run(pkg, gpu, qkv, lens)
+    assert np.abs(got - oracle.fmha(qkv, lens)).max() <= TOL_F16
+    qkv = make_qkv(rng, 8, 512, 16)
     got = run(pkg, gpu, qkv, lens)
     assert excess(got, oracle.fmha(qkv, lens), TOL_F16) <= 1.0
 
