@@ -10,8 +10,11 @@ and reported under "kernels" in the same JSON line, each against the roofline
 that bounds it.
 
 Timing: K launches are enqueued back to back on one stream between two HIP
-events recorded on that same stream (captured into one hipGraph so the host
-launch cost does not throttle microsecond kernels).  Memory-bound kernels rotate
+events recorded on that same stream.  The calls are made from a C++ loop
+(lib/libmgpu_bench_loops.so, K calls of the same C-ABI entry point a compiled
+model calls) because a ctypes call costs more host time than a streaming
+kernel runs; --graph times a hipGraph of K ctypes launches instead and gives
+the same figures within a few per cent.  Memory-bound kernels rotate
 through enough distinct buffer sets (> 256 MiB in total) that no launch finds
 its operands in the Infinity Cache left by an earlier one; the cache-resident
 ("warm") figure is reported next to it.
@@ -23,6 +26,7 @@ target.
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -48,7 +52,9 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-graph", action="store_true", help="enqueue launches directly instead of through a hipGraph")
+    ap.add_argument("--graph", action="store_true",
+                    help="time a hipGraph of K ctypes launches instead of the C++ launch loops")
+    ap.add_argument("--no-graph", action="store_true", help="with --graph: enqueue the ctypes launches directly")
     ap.add_argument("--only", type=str, default="", help="comma list of kernels to run besides the headline")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run plain device copies of 64 MiB (for scaling FETCH_SIZE / WRITE_SIZE counters)")
@@ -136,6 +142,23 @@ def main():
     torch.cuda.set_device(dev)
     lib = pkg.ops()
     timer = Timer(torch, use_graph=not args.no_graph)
+    loops = None
+    if not args.graph:
+        # K calls of the C-ABI entry point from a C++ loop between two events on
+        # the launch stream (lib/libmgpu_bench_loops.so): the call rate of a
+        # compiled model, which a Python caller cannot reach
+        loops = ctypes.CDLL(os.path.join(pkg.LIB_DIR, "libmgpu_bench_loops.so"))
+        for fn in ("mgpuBenchLayerNormF32", "mgpuBenchLayerNormF16", "mgpuBenchAddF32", "mgpuBenchFusedMHAF16"):
+            getattr(loops, fn).restype = ctypes.c_float
+    bench_stream = torch.cuda.Stream()
+
+    def ptrs(tensors):
+        return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+    def loop_ms(ms):
+        if ms < 0:
+            raise RuntimeError("timed launch loop failed")
+        return ms
     K, W = args.steps, args.warmup
     only = set(filter(None, args.only.split(",")))
 
@@ -175,9 +198,15 @@ def main():
         lib.mgpuLayerNormF32(xs[i % len(xs)].data_ptr(), gamma.data_ptr(), beta.data_ptr(),
                              ys[i % len(ys)].data_ptr(), 1e-5, m, n, s)
 
-    ms_cold = timer.run(ln32, K, W)
-    check()
-    ms_warm = timer.run(lambda i: ln32(0), K, W)
+    if loops:
+        torch.cuda.synchronize()
+        sp = ctypes.c_void_p(bench_stream.cuda_stream)
+        ln_args = (ctypes.c_void_p(gamma.data_ptr()), ctypes.c_void_p(beta.data_ptr()), ctypes.c_float(1e-5), m, n)
+        ms_cold = loop_ms(loops.mgpuBenchLayerNormF32(ptrs(xs), ptrs(ys), nsets, *ln_args, K, W, sp))
+        ms_warm = loop_ms(loops.mgpuBenchLayerNormF32(ptrs(xs[:1]), ptrs(ys[:1]), 1, *ln_args, K, W, sp))
+    else:
+        ms_cold = timer.run(ln32, K, W)
+        ms_warm = timer.run(lambda i: ln32(0), K, W)
     check()
     headline = hbm_entry("layernorm_f32", "LayerNorm fp32 (32,128,768) eps=1e-5 [configs[1]]", "f32",
                          ln_bytes, ms_cold, K, ms_warm)
@@ -196,8 +225,14 @@ def main():
             lib.mgpuLayerNormF16(xh[i % nsets].data_ptr(), gh.data_ptr(), bh.data_ptr(),
                                  yh[i % nsets].data_ptr(), 1e-5, m, n, s)
 
-        ms = timer.run(ln16, K, W)
-        msw = timer.run(lambda i: ln16(0), K, W)
+        if loops:
+            torch.cuda.synchronize()
+            a16 = (ctypes.c_void_p(gh.data_ptr()), ctypes.c_void_p(bh.data_ptr()), ctypes.c_float(1e-5), m, n)
+            ms = loop_ms(loops.mgpuBenchLayerNormF16(ptrs(xh), ptrs(yh), nsets, *a16, K, W, sp))
+            msw = loop_ms(loops.mgpuBenchLayerNormF16(ptrs(xh[:1]), ptrs(yh[:1]), 1, *a16, K, W, sp))
+        else:
+            ms = timer.run(ln16, K, W)
+            msw = timer.run(lambda i: ln16(0), K, W)
         check()
         kernels.append(hbm_entry("layernorm_f16", "LayerNorm fp16 (32,128,768)", "f16",
                                  2 * m * n * 2 + 2 * n * 2, ms, K, msw))
@@ -216,8 +251,13 @@ def main():
             j = i % nsets
             lib.mgpuAddF32(aa[j].data_ptr(), bb[j].data_ptr(), cc[j].data_ptr(), ne, s)
 
-        ms = timer.run(add, K, W)
-        msw = timer.run(lambda i: add(0), K, W)
+        if loops:
+            torch.cuda.synchronize()
+            ms = loop_ms(loops.mgpuBenchAddF32(ptrs(aa), ptrs(bb), ptrs(cc), nsets, ctypes.c_int64(ne), K, W, sp))
+            msw = loop_ms(loops.mgpuBenchAddF32(ptrs(aa[:1]), ptrs(bb[:1]), ptrs(cc[:1]), 1, ctypes.c_int64(ne), K, W, sp))
+        else:
+            ms = timer.run(add, K, W)
+            msw = timer.run(lambda i: add(0), K, W)
         check()
         kernels.append(hbm_entry("add_f32", "add fp32 (3,640,640) [configs[0]]", "f32", 3 * ne * 4, ms, K, msw))
         del aa, bb, cc
@@ -242,7 +282,13 @@ def main():
                                 out.data_ptr(), B, S, H, D, 0.125, 0, s)
 
         steps = max(20, K // 4)
-        ms = timer.run(run, steps, max(3, W // 4))
+        if loops:
+            torch.cuda.synchronize()
+            ms = loop_ms(loops.mgpuBenchFusedMHAF16(
+                ptrs([qkv]), ptrs([out]), 1, ctypes.c_void_p(lens.data_ptr() if lens is not None else None),
+                B, S, H, D, ctypes.c_float(0.125), 0, steps, max(3, W // 4), sp))
+        else:
+            ms = timer.run(run, steps, max(3, W // 4))
         check()
         us = ms * 1e3 / steps
         tf = flop_valid / us / 1e6
@@ -319,7 +365,8 @@ def main():
         "ms_per_step": round(ms_cold / K, 6), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": headline["workload"], "rows": m, "cols": n, "eps": 1e-5,
-                   "launch_mode": "direct" if args.no_graph else "hipGraph of K launches",
+                   "launch_mode": ("C++ loop of K calls of the C-ABI entry point" if loops else
+                                   "direct ctypes launches" if args.no_graph else "hipGraph of K ctypes launches"),
                    "buffer_sets": rotating_sets(2 * m * n * 4)},
         "roofline": headline["roofline"], "cache_resident": headline.get("cache_resident"),
         "cpu_baseline": cpu, "kernels": kernels,

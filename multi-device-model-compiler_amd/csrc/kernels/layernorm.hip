@@ -21,8 +21,10 @@ namespace {
 constexpr int kMaxVPL = 8; // vectors per lane the register kernel is built for
 
 // One group of LANES lanes owns one row: lane l holds vectors l, l+LANES, ...
-// (VPL of them, the last ones predicated off when the row is shorter).
-template <typename T, int LANES, int VPL, bool RESIDUAL>
+// (VPL of them, the last ones predicated off when the row is shorter; FULL
+// says that the row fills all of them, which removes every predicate and with
+// it the branches that would sit between the loads).
+template <typename T, int LANES, int VPL, bool RESIDUAL, bool FULL>
 __global__ __launch_bounds__(256) void layernorm_rows_kernel(
     const T *__restrict__ input, const T *__restrict__ residual, const T *__restrict__ gamma,
     const T *__restrict__ beta, T *__restrict__ sumOut, T *__restrict__ normed, float eps, int m,
@@ -35,8 +37,21 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
   const int nvec = n / VEC;
   const float inv_n = 1.0f / (float)n;
 
+  // gamma and beta do not depend on the row: fetch them once, ahead of the row
+  // data, so that their latency is not paid between the reductions and the
+  // stores (a wavefront usually owns a single row and its run time is one
+  // chain of latencies).
   const u32x4 *gv = reinterpret_cast<const u32x4 *>(gamma);
   const u32x4 *bv = reinterpret_cast<const u32x4 *>(beta);
+  u32x4 graw[VPL], braw[VPL];
+#pragma unroll
+  for (int k = 0; k < VPL; k++) {
+    const int v = lane + k * LANES;
+    if (FULL || v < nvec) {
+      graw[k] = gv[v];
+      braw[k] = bv[v];
+    }
+  }
 
   for (int row = blockIdx.x * GROUPS + group; row < m; row += gridDim.x * GROUPS) {
     const u32x4 *xv = reinterpret_cast<const u32x4 *>(input + (size_t)row * n);
@@ -46,7 +61,7 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
 #pragma unroll
     for (int k = 0; k < VPL; k++) {
       const int v = lane + k * LANES;
-      if (v < nvec) {
+      if (FULL || v < nvec) {
         raw[k] = xv[v];
         if (RESIDUAL) rawr[k] = rv[v];
       }
@@ -57,7 +72,7 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
 #pragma unroll
     for (int k = 0; k < VPL; k++) {
       const int v = lane + k * LANES;
-      if (v < nvec) {
+      if (FULL || v < nvec) {
         Tr::unpack(raw[k], x[k]);
         if (RESIDUAL) {
           float r[VEC];
@@ -78,7 +93,7 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
 #pragma unroll
     for (int k = 0; k < VPL; k++) {
       const int v = lane + k * LANES;
-      if (v < nvec) {
+      if (FULL || v < nvec) {
 #pragma unroll
         for (int e = 0; e < VEC; e++) {
           const float d = x[k][e] - mean;
@@ -94,10 +109,10 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
 #pragma unroll
     for (int k = 0; k < VPL; k++) {
       const int v = lane + k * LANES;
-      if (v < nvec) {
+      if (FULL || v < nvec) {
         float g[VEC], b[VEC], y[VEC];
-        Tr::unpack(gv[v], g);
-        Tr::unpack(bv[v], b);
+        Tr::unpack(graw[k], g);
+        Tr::unpack(braw[k], b);
         if (RESIDUAL) {
           // The sum is stored rounded to T and the normalised value is taken
           // from that rounded sum, while mean and variance came from the
@@ -171,8 +186,12 @@ void launchRows(const T *input, const T *residual, const T *gamma, const T *beta
   int64_t blocks = ((int64_t)m + GROUPS - 1) / GROUPS;
   const int64_t cap = (int64_t)numComputeUnits() * 8;
   if (blocks > cap) blocks = cap;
-  layernorm_rows_kernel<T, LANES, VPL, RESIDUAL><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
-      input, residual, gamma, beta, sumOut, normed, eps, m, n);
+  if (n / ElemTraits<T>::kVec == LANES * VPL)
+    layernorm_rows_kernel<T, LANES, VPL, RESIDUAL, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+        input, residual, gamma, beta, sumOut, normed, eps, m, n);
+  else
+    layernorm_rows_kernel<T, LANES, VPL, RESIDUAL, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+        input, residual, gamma, beta, sumOut, normed, eps, m, n);
   MGPU_CHECK_LAUNCH("layernorm_rows_kernel");
 }
 
