@@ -262,6 +262,29 @@ def main():
         kernels.append(hbm_entry("add_f32", "add fp32 (3,640,640) [configs[0]]", "f32", 3 * ne * 4, ms, K, msw))
         del aa, bb, cc
 
+    # ---------------- the same two kernels where launch latency is amortised ----
+    # (the configurations above move 15-25 MB per launch, a few microseconds of
+    # HBM time; these move 1.6 GB and 3.2 GB)
+    if want("layernorm_f32_large") and loops:
+        mL = 64 * m
+        xl = torch.randn((mL, n), device=dev, generator=gen)
+        yl = torch.empty_like(xl)
+        torch.cuda.synchronize()
+        ms = loop_ms(loops.mgpuBenchLayerNormF32(ptrs([xl]), ptrs([yl]), 1, *ln_args[:3], mL, n, 20, 3, sp))
+        check()
+        kernels.append(hbm_entry("layernorm_f32_large", f"LayerNorm fp32 ({mL},{n})", "f32",
+                                 2 * mL * n * 4 + 2 * n * 4, ms, 20))
+        del xl, yl
+    if want("add_f32_large") and loops:
+        nl = 1 << 28
+        al, bl = torch.rand(nl, device=dev, generator=gen), torch.rand(nl, device=dev, generator=gen)
+        cl = torch.empty_like(al)
+        torch.cuda.synchronize()
+        ms = loop_ms(loops.mgpuBenchAddF32(ptrs([al]), ptrs([bl]), ptrs([cl]), 1, ctypes.c_int64(nl), 20, 3, sp))
+        check()
+        kernels.append(hbm_entry("add_f32_large", f"add fp32 ({nl} elements)", "f32", 3 * nl * 4, ms, 20))
+        del al, bl, cl
+
     # ---------------- fused MHA -------------------------------------------------
     def fmha_case(name, workload, B, S, H, masked):
         D = 64

@@ -56,12 +56,11 @@ void addF32(const float *a, const float *b, float *c, int64_t n, hipStream_t str
   if (n < 0) fail("mgpuAddF32: negative element count");
   if (n == 0) return;
   if (!a || !b || !c) fail("mgpuAddF32: null pointer");
-  const int cus = numComputeUnits();
   if (aligned16(a) && aligned16(b) && aligned16(c) && n >= 4) {
     constexpr int UNROLL = 1;
     const int64_t n4 = n / 4;
     int64_t blocks = (n4 + 256 * UNROLL - 1) / (256 * UNROLL);
-    const int64_t cap = (int64_t)cus * 16;
+    const int64_t cap = kMaxStreamBlocks;
     if (blocks > cap) blocks = cap;
     add_f32_vec4_kernel<UNROLL><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
         reinterpret_cast<const float4v *>(a), reinterpret_cast<const float4v *>(b),
@@ -73,7 +72,7 @@ void addF32(const float *a, const float *b, float *c, int64_t n, hipStream_t str
     }
   } else {
     int64_t blocks = (n + 255) / 256;
-    const int64_t cap = (int64_t)cus * 16;
+    const int64_t cap = kMaxStreamBlocks;
     if (blocks > cap) blocks = cap;
     add_f32_scalar_kernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(a, b, c, 0, n);
     MGPU_CHECK_LAUNCH("add_f32_scalar_kernel");

@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void fill_kernel(T *__restrict__ dst, size_t n
 
 unsigned gridFor(size_t items, int perBlock) {
   size_t blocks = (items + perBlock - 1) / perBlock;
-  const size_t cap = (size_t)numComputeUnits() * 16;
+  const size_t cap = (size_t)kMaxStreamBlocks;
   if (blocks > cap) blocks = cap;
   if (blocks == 0) blocks = 1;
   return (unsigned)blocks;

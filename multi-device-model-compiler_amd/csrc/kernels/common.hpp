@@ -31,6 +31,14 @@ inline void checkHipStatus(hipError_t status, const char *where) {
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Streaming kernels get one block per block-sized piece of the array rather
+// than a grid sized to the machine with a stride loop: blocks are dispatched
+// in index order, so at any moment the whole device works on one contiguous
+// window of memory, which the HBM controllers serve faster (6.4 against
+// 4.5-5.7 TB/s measured on a 1 GiB copy).  The stride loop only takes over
+// beyond this many blocks.
+constexpr int64_t kMaxStreamBlocks = int64_t(1) << 22;
+
 inline int numComputeUnits() {
   static int cus = [] {
     int dev = 0, v = 0;

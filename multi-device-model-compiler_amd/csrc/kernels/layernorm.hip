@@ -184,7 +184,7 @@ void launchRows(const T *input, const T *residual, const T *gamma, const T *beta
                 T *normed, float eps, int m, int n, hipStream_t stream) {
   constexpr int GROUPS = 256 / LANES;
   int64_t blocks = ((int64_t)m + GROUPS - 1) / GROUPS;
-  const int64_t cap = (int64_t)numComputeUnits() * 8;
+  const int64_t cap = kMaxStreamBlocks;
   if (blocks > cap) blocks = cap;
   if (n / ElemTraits<T>::kVec == LANES * VPL)
     layernorm_rows_kernel<T, LANES, VPL, RESIDUAL, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
@@ -240,7 +240,7 @@ void layerNormTyped(const T *input, const T *residual, const T *gamma, const T *
     return;
   }
   int64_t blocks = m;
-  const int64_t cap = (int64_t)numComputeUnits() * 8;
+  const int64_t cap = kMaxStreamBlocks;
   if (blocks > cap) blocks = cap;
   layernorm_general_kernel<T, RESIDUAL><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
       input, residual, gamma, beta, sumOut, normed, eps, m, n);

@@ -57,7 +57,10 @@ def test_matmul_ex_f16_epilogues(pkg, gpu, oracle, rng, M, K, N):
                     (dict(bias=tb, residual=tr), dict(bias=b, residual=r))]:
         got = pkg.matmul_ex(tx, tw, **kw).cpu().numpy().astype(np.float32)
         ref = oracle.gemm(x, w, **okw)
-        assert np.all(np.abs(got - ref) <= f16_tol(ref)), (kw.keys(), np.abs(got - ref).max())
+        # GELU runs on the fp16-rounded GEMM output: two roundings, and the first is taken
+        # at the pre-activation magnitude, which can sit one binade above the result
+        k_ulp = 2.5 if kw.get("act") == pkg.ACT_GELU else 1.0
+        assert np.all(np.abs(got - ref) <= f16_tol(ref, k_ulp)), (kw.keys(), np.abs(got - ref).max())
 
 
 def test_matmul_f32(pkg, gpu, oracle, rng):
