@@ -286,8 +286,7 @@ def main():
         del al, bl, cl
 
     # ---------------- fused MHA -------------------------------------------------
-    def fmha_case(name, workload, B, S, H, masked):
-        D = 64
+    def fmha_case(name, workload, B, S, H, masked, D=64):
         qkv = (torch.randn((B, S, 3, H, D), device=dev, generator=gen) / 8).half()
         out = torch.empty((B, S, H * D), device=dev, dtype=torch.float16)
         lens = None
@@ -302,14 +301,14 @@ def main():
         def run(i):
             s = torch.cuda.current_stream().cuda_stream
             lib.mgpuFusedMHAF16(qkv.data_ptr(), lens.data_ptr() if lens is not None else None,
-                                out.data_ptr(), B, S, H, D, 0.125, 0, s)
+                                out.data_ptr(), B, S, H, D, D ** -0.5, 0, s)
 
         steps = max(20, K // 4)
         if loops:
             torch.cuda.synchronize()
             ms = loop_ms(loops.mgpuBenchFusedMHAF16(
                 ptrs([qkv]), ptrs([out]), 1, ctypes.c_void_p(lens.data_ptr() if lens is not None else None),
-                B, S, H, D, ctypes.c_float(0.125), 0, steps, max(3, W // 4), sp))
+                B, S, H, D, ctypes.c_float(D ** -0.5), 0, steps, max(3, W // 4), sp))
         else:
             ms = timer.run(run, steps, max(3, W // 4))
         check()
@@ -333,6 +332,10 @@ def main():
                   8, 512, 16, True)
     if want("fmha_b32_s512"):
         fmha_case("fmha_b32_s512", "fused MHA fp16 b32 s512 h12 d64 [roofline target shape]", 32, 512, 12, False)
+
+    if want("fmha_d128_b32_s512"):
+        fmha_case("fmha_d128_b32_s512", "fused MHA fp16 b32 s512 h8 d128 [the reference layer's head geometry]",
+                  32, 512, 8, False, D=128)
 
     # ---------------- BERT-base encoder layer ----------------------------------
     if want("bert_layer"):

@@ -85,7 +85,7 @@ void mgpuAddResidualPreLayerNormBF16(const void *input, const void *residual, co
 
 /* ---- fused multi-head attention -------------------------------------- */
 /* out[b,i,h,:] = sum_j softmax_j(scale * <q[b,i,h,:], k[b,j,h,:]>) v[b,j,h,:]
- * qkv: packed [B, S, 3, H, D]; out: [B, S, H*D]; D must be 64.
+ * qkv: packed [B, S, 3, H, D]; out: [B, S, H*D]; D is 64 or 128.
  * seqlens: NULL, or B int32 valid key counts (keys j >= seqlens[b] are masked
  * out; all S query rows are produced).  causal != 0 also masks j > i.
  * No score matrix is written to memory.

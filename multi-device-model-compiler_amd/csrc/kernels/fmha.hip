@@ -1,4 +1,4 @@
-// Fused multi-head attention forward for head_dim 64 on gfx950 MFMA.
+// Fused multi-head attention forward for head_dim 64 and 128 on gfx950 MFMA.
 //
 // Replaces the cubin kernels the reference dispatches through
 // FusedMHARunnerFP16v2 (3rdparty/trt_fused_multihead_attention/
@@ -9,7 +9,8 @@
 //
 // Work decomposition.  A 256-thread block (4 wavefronts) owns BM = 128 * NQ
 // consecutive queries of one (batch, head); each wavefront owns NQ blocks of 32
-// queries.  Key/value tiles of BN = 64 keys travel HBM -> LDS directly
+// queries.  Key/value tiles of 8 KiB (64 keys at head_dim 64, 32 keys at 128;
+// the comments below give the head_dim 64 numbers) travel HBM -> LDS directly
 // (global_load_lds, 16 bytes per lane, no register staging) into a ring of
 // three LDS stages shared by the 4 wavefronts, so two tiles are always in
 // flight behind the one being consumed.
@@ -75,11 +76,27 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef unsigned char __attribute__((address_space(3))) lds_u8; // a byte in LDS
 
-constexpr int kD = 64;   // head dim
-constexpr int kBN = 64;  // keys per tile
-constexpr int kStages = 3;               // LDS ring depth
-constexpr int kTileBytes = kBN * kD * 2; // one K or V tile: 64 rows of 128 B, unpadded
-constexpr int kOS = 68;  // output staging row stride in elements
+// Geometry per head dimension D (64 or 128).  A K or V tile is always 8 KiB:
+// 64 keys of 128 bytes or 32 keys of 256 bytes, so both share the ring, the
+// movers and the MFMA count per tile (8 for the scores, 8 for P.V); at D = 128
+// a tile carries half as many scores, i.e. half the softmax work per MFMA.
+constexpr int kStages = 3;        // LDS ring depth
+constexpr int kTileBytes = 8192;  // one K or V tile, unpadded rows
+template <int D> struct Geo {
+  static_assert(D == 64 || D == 128, "head dimension 64 or 128");
+  static constexpr int kBN = kTileBytes / (D * 2); // keys per tile: 64 / 32
+  static constexpr int KB = kBN / 32;              // 32-key score blocks per tile: 2 / 1
+  static constexpr int DC = D / 16;                // MFMA k-steps over the head dimension: 4 / 8
+  static constexpr int DB = D / 32;                // 32-row blocks of O^T: 2 / 4
+  static constexpr int rowBytes = D * 2;           // 128 / 256
+  static constexpr int CPR = rowBytes / 16;        // 16-byte chunks per row: 8 / 16
+  static constexpr int RPI = 64 / CPR;             // tile rows one wavefront load instruction fills: 8 / 4
+  static constexpr int OS = D + 4;                 // output staging row stride in elements
+  // chunk swizzles (XOR on the 16-byte chunk index of a row) that keep the K
+  // operand reads and the transposing V reads free of bank conflicts
+  __host__ __device__ static constexpr int kSwz(int row) { return D == 64 ? ((row >> 1) & 7) : (row & 15); }
+  __host__ __device__ static constexpr int vSwz(int row) { return D == 64 ? (((row >> 1) & 1) << 2) : ((row & 3) << 2); }
+};
 constexpr float kSumLimit = 1e30f; // a row sum above this (or NaN) means P overflowed against the stale m
 
 template <typename T> struct Mma;
@@ -134,15 +151,17 @@ __device__ __forceinline__ float halves_sum(float v) {
   return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
 }
 
-template <typename T, int NQ, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__restrict__ qkv,
+template <typename T, int D, int NQ, bool CAUSAL>
+__global__ __launch_bounds__(256, 2) void fmha_fwd_kernel(const uint16_t *__restrict__ qkv,
                                                               const int32_t *__restrict__ seqlens,
                                                               uint16_t *__restrict__ out, int S, int H,
                                                               int nQB, float scale_log2e) {
   using M = Mma<T>;
   using v8 = typename M::v8;
   using v4 = typename M::v4;
+  using G = Geo<D>;
   constexpr int BM = 128 * NQ;
+  constexpr int kD = D, kBN = G::kBN;
 
   // Ring of kStages stages, each a K tile followed by a V tile; reused as the
   // output staging area at the end.
@@ -186,17 +205,16 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
   const int nkt = (kend + kBN - 1) / kBN;
 
   // ---- tile movers: HBM -> LDS, 16 bytes per lane ---------------------------
-  // One wavefront instruction fills 1 KiB = 8 tile rows; wavefront w moves rows
-  // 16w .. 16w+15 of both tiles.  Lane l lands in LDS chunk l%8 of row l/8 and
-  // fetches global chunk (l%8) ^ swizzle(row): swizzle = (row/2)%8 for K,
-  // 4*((row/2)%2) for V.
-  const int mrow = lane / 8, mchunk = lane % 8;
+  // One wavefront instruction fills 1 KiB = RPI tile rows; wavefront w moves
+  // 2 KiB of both tiles.  Lane l lands in LDS chunk l % CPR of row l / CPR and
+  // fetches global chunk (l % CPR) ^ swizzle(row).
+  const int mrow = lane / G::CPR, mchunk = lane % G::CPR;
   uint32_t koff[2], voff[2];
 #pragma unroll
   for (int i = 0; i < 2; i++) {
-    const int row = 8 * (2 * wave + i) + mrow;
-    koff[i] = (uint32_t)row * tokBytes + (uint32_t)((mchunk ^ ((row >> 1) & 7)) * 16);
-    voff[i] = (uint32_t)row * tokBytes + (uint32_t)((mchunk ^ (((row >> 1) & 1) << 2)) * 16);
+    const int row = G::RPI * (2 * wave + i) + mrow;
+    koff[i] = (uint32_t)row * tokBytes + (uint32_t)((mchunk ^ G::kSwz(row)) * 16);
+    voff[i] = (uint32_t)row * tokBytes + (uint32_t)((mchunk ^ G::vSwz(row)) * 16);
   }
   // The loads are written as inline assembly so that the compiler's wait-count
   // bookkeeping does not see them: it would otherwise wait for every load in
@@ -223,12 +241,12 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
     } else { // last tile of a ragged sequence: clamp the row, the mask hides it
 #pragma unroll
       for (int i = 0; i < 2; i++) {
-        const int row = 8 * (2 * wave + i) + mrow;
+        const int row = G::RPI * (2 * wave + i) + mrow;
         int key = kt * kBN + row;
         key = key < S ? key : S - 1;
-        const uint32_t rowBytes = (uint32_t)key * tokBytes;
-        dma16(rowBytes + (mchunk ^ ((row >> 1) & 7)) * 16, kbase, kdst + i * 1024);
-        dma16(rowBytes + (mchunk ^ (((row >> 1) & 1) << 2)) * 16, vbase, vdst + i * 1024);
+        const uint32_t rowOff = (uint32_t)key * tokBytes;
+        dma16(rowOff + (mchunk ^ G::kSwz(row)) * 16, kbase, kdst + i * 1024);
+        dma16(rowOff + (mchunk ^ G::vSwz(row)) * 16, vbase, vdst + i * 1024);
       }
     }
   };
@@ -239,41 +257,41 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
     if (t < nkt) issueTile(t);
 
   // Q as the B operand: lane (query l32, k-slots = d 16c + 8hl .. +7).
-  v8 qf[NQ][4];
+  v8 qf[NQ][G::DC];
 #pragma unroll
   for (int qi = 0; qi < NQ; qi++) {
     int row = q0 + qi * 32 + l32;
     row = row < S ? row : S - 1;
 #pragma unroll
-    for (int c = 0; c < 4; c++)
+    for (int c = 0; c < G::DC; c++)
       qf[qi][c] = *reinterpret_cast<const v8 *>(qbase + (size_t)row * tokBytes + (16 * c + 8 * hl) * 2);
   }
 
   // ---- operand addresses inside a stage ---------------------------------------
   // K: lane (key l32 [+32kb], d chunk 2c+hl) reads 16 bytes.
-  uint32_t kfrag[4];
+  uint32_t kfrag[G::DC];
 #pragma unroll
-  for (int c = 0; c < 4; c++) kfrag[c] = (uint32_t)(l32 * 128 + (((2 * c + hl) ^ ((l32 >> 1) & 7)) * 16));
+  for (int c = 0; c < G::DC; c++) kfrag[c] = (uint32_t)(l32 * G::rowBytes + (((2 * c + hl) ^ G::kSwz(l32)) * 16));
   // V: as a source of the transposing read, lane L of a 16-lane group g points
   // at key 4*hl + L/4 (+ 32kb + 16m + 8e), d = 32db + 16*(g%2) + 4*(L%4).
-  uint32_t vfrag[2];
+  uint32_t vfrag[G::DB];
   {
-    const int g = lane / 16, L = lane % 16, r = L % 4, j = L / 4, jb = (j >> 1) & 1;
+    const int g = lane / 16, L = lane % 16, r = L % 4, j = L / 4;
 #pragma unroll
-    for (int db = 0; db < 2; db++) {
-      const int chunk = (4 * db + 2 * (g % 2) + r / 2) ^ (jb << 2);
-      vfrag[db] = (uint32_t)((4 * hl + j) * 128 + chunk * 16 + 8 * (r % 2));
+    for (int db = 0; db < G::DB; db++) {
+      const int chunk = (4 * db + 2 * (g % 2) + r / 2) ^ G::vSwz(4 * hl + j);
+      vfrag[db] = (uint32_t)((4 * hl + j) * G::rowBytes + chunk * 16 + 8 * (r % 2));
     }
   }
 
-  f32x16 accO[NQ][2];
+  f32x16 accO[NQ][G::DB];
   float m_run[NQ], l_run[NQ]; // stale reference maximum (raw score units), running sum
 #pragma unroll
   for (int qi = 0; qi < NQ; qi++) {
     m_run[qi] = -INFINITY;
     l_run[qi] = 0.0f;
 #pragma unroll
-    for (int db = 0; db < 2; db++)
+    for (int db = 0; db < G::DB; db++)
 #pragma unroll
       for (int i = 0; i < 16; i++) accO[qi][db][i] = 0.0f;
   }
@@ -297,7 +315,7 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
 #pragma unroll
       for (int i = 0; i < 2; i++) {
         const int chunk = tid + 256 * i; // 16-byte chunk of the V tile
-        if (key0 + chunk / 8 >= kvlen)
+        if (key0 + chunk / G::CPR >= kvlen)
           *reinterpret_cast<u32x4 *>(vst + chunk * 16) = u32x4{0u, 0u, 0u, 0u};
       }
       __syncthreads();
@@ -308,20 +326,20 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
 
     // Operand pointers in the LDS address space: one add per tile, the rest
     // of every address is an instruction immediate.
-    const lds_u8 *kp[4], *vp[2];
+    const lds_u8 *kp[G::DC], *vp[G::DB];
 #pragma unroll
-    for (int c = 0; c < 4; c++) kp[c] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kfrag[c]);
+    for (int c = 0; c < G::DC; c++) kp[c] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kfrag[c]);
 #pragma unroll
-    for (int db = 0; db < 2; db++) vp[db] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kTileBytes + vfrag[db]);
+    for (int db = 0; db < G::DB; db++) vp[db] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kTileBytes + vfrag[db]);
 
     // ---- S^T = K Q^T -------------------------------------------------------
-    f32x16 accS[NQ][2];
+    f32x16 accS[NQ][G::KB];
     __builtin_amdgcn_s_setprio(2); // MFMA phases outrank the softmax phases of the SIMD's other wavefronts
 #pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
+    for (int kb = 0; kb < G::KB; kb++) {
 #pragma unroll
-      for (int c = 0; c < 4; c++) {
-        const v8 a = *reinterpret_cast<const v8 __attribute__((address_space(3))) *>(kp[c] + kb * 4096);
+      for (int c = 0; c < G::DC; c++) {
+        const v8 a = *reinterpret_cast<const v8 __attribute__((address_space(3))) *>(kp[c] + kb * 32 * G::rowBytes);
 #pragma unroll
         for (int qi = 0; qi < NQ; qi++) {
           if (c == 0) {
@@ -335,13 +353,13 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
 
     __builtin_amdgcn_s_setprio(0);
     const bool needMask = (key0 + kBN > kvlen) || (CAUSAL && key0 + kBN - 1 > q0);
-    v8 pf[NQ][2][2];
+    v8 pf[NQ][G::KB][2];
 #pragma unroll
     for (int qi = 0; qi < NQ; qi++) {
       if (needMask) {
         const int query = q0 + qi * 32 + l32;
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
+        for (int kb = 0; kb < G::KB; kb++)
 #pragma unroll
           for (int i = 0; i < 16; i++) {
             const int key = key0 + 32 * kb + 8 * (i / 4) + 4 * hl + (i % 4);
@@ -354,7 +372,7 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
         const float mc = mref * scale_log2e;
         float lsum = 0.0f;
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
+        for (int kb = 0; kb < G::KB; kb++)
 #pragma unroll
           for (int m = 0; m < 2; m++) {
 #pragma unroll
@@ -370,7 +388,7 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
       if (__builtin_amdgcn_ballot_w64(!(lsum <= kSumLimit)) != 0) {
         float mx = accS[qi][0][0];
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
+        for (int kb = 0; kb < G::KB; kb++)
 #pragma unroll
           for (int i = 0; i < 16; i++) mx = fmaxf(mx, accS[qi][kb][i]);
         mx = halves_max(mx);
@@ -380,7 +398,7 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
         m_run[qi] = m_new;
         l_run[qi] *= alpha;
 #pragma unroll
-        for (int db = 0; db < 2; db++)
+        for (int db = 0; db < G::DB; db++)
 #pragma unroll
           for (int i = 0; i < 16; i++) accO[qi][db][i] *= alpha;
         lsum = makeP(m_new);
@@ -391,14 +409,14 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
     // ---- O^T += V^T P^T ----------------------------------------------------
     __builtin_amdgcn_s_setprio(2);
 #pragma unroll
-    for (int db = 0; db < 2; db++) {
+    for (int db = 0; db < G::DB; db++) {
 #pragma unroll
-      for (int kb = 0; kb < 2; kb++) {
+      for (int kb = 0; kb < G::KB; kb++) {
 #pragma unroll
         for (int m = 0; m < 2; m++) {
-          const lds_u8 *p = vp[db] + (32 * kb + 16 * m) * 128;
-          const v4 lo = M::readTr(p);            // k-slots 0..3: keys +4hl+0..3
-          const v4 hi = M::readTr(p + 8 * 128);  // k-slots 4..7: keys +8+4hl+0..3
+          const lds_u8 *p = vp[db] + (32 * kb + 16 * m) * G::rowBytes;
+          const v4 lo = M::readTr(p);                    // k-slots 0..3: keys +4hl+0..3
+          const v4 hi = M::readTr(p + 8 * G::rowBytes);  // k-slots 4..7: keys +8+4hl+0..3
           const v8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
           for (int qi = 0; qi < NQ; qi++) accO[qi][db] = M::run(a, pf[qi][kb][m], accO[qi][db]);
@@ -410,6 +428,7 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
 
   // ---- normalise, transpose through LDS, store whole rows ------------------
   __syncthreads(); // every wavefront is done reading the K / V tiles
+  constexpr int kOS = G::OS;
   uint16_t *stage = reinterpret_cast<uint16_t *>(smem) + wave * (NQ * 32 * kOS);
   static_assert(4 * NQ * 32 * kOS * 2 <= kStages * 2 * kTileBytes, "output staging must fit in the ring");
 #pragma unroll
@@ -417,7 +436,7 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
     const float l = halves_sum(l_run[qi]);
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
 #pragma unroll
-    for (int db = 0; db < 2; db++)
+    for (int db = 0; db < G::DB; db++)
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         v4 o;
@@ -429,9 +448,9 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
   // Each wavefront reads back only what it wrote: no block barrier needed, the
   // LDS accesses of one wavefront are ordered.
 #pragma unroll
-  for (int it = 0; it < NQ * 4; it++) {
+  for (int it = 0; it < NQ * 32 * G::CPR / 64; it++) {
     const int chunk = it * 64 + lane; // 16-byte chunk index inside the wave's tile
-    const int r = chunk / 8, cidx = chunk % 8;
+    const int r = chunk / G::CPR, cidx = chunk % G::CPR;
     const int query = q0 + r;
     if (query < S) {
       // 8-byte LDS reads: the staging stride is 8-byte but not 16-byte aligned
@@ -444,7 +463,7 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_d64_kernel(const uint16_t *__
   }
 }
 
-template <typename T, int NQ>
+template <typename T, int D, int NQ>
 void launch(const void *qkv, const int32_t *seqlens, void *out, int B, int S, int H, float scale,
             bool causal, hipStream_t stream) {
   constexpr int BM = 128 * NQ;
@@ -455,10 +474,10 @@ void launch(const void *qkv, const int32_t *seqlens, void *out, int B, int S, in
   const auto *in = static_cast<const uint16_t *>(qkv);
   auto *o = static_cast<uint16_t *>(out);
   if (causal)
-    fmha_fwd_d64_kernel<T, NQ, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, o, S, H, nQB, c);
+    fmha_fwd_kernel<T, D, NQ, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, o, S, H, nQB, c);
   else
-    fmha_fwd_d64_kernel<T, NQ, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, o, S, H, nQB, c);
-  MGPU_CHECK_LAUNCH("fmha_fwd_d64_kernel");
+    fmha_fwd_kernel<T, D, NQ, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, o, S, H, nQB, c);
+  MGPU_CHECK_LAUNCH("fmha_fwd_kernel");
 }
 
 } // namespace
@@ -466,19 +485,21 @@ void launch(const void *qkv, const int32_t *seqlens, void *out, int B, int S, in
 void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int B, int S, int H,
               int D, float scale, bool causal, hipStream_t stream) {
   if (B < 0 || S < 0 || H < 0) fail("fusedMHA: negative shape");
-  if (D != kD) fail("fusedMHA: only head_dim 64 is built");
+  if (D != 64 && D != 128) fail("fusedMHA: head_dim must be 64 or 128");
   if (B == 0 || S == 0 || H == 0) return;
   if (!qkv || !out) fail("fusedMHA: null pointer");
   if (!aligned16(qkv) || !aligned16(out)) fail("fusedMHA: qkv and out must be 16-byte aligned");
   if (!(scale > 0.0f) || !(scale < INFINITY)) fail("fusedMHA: softmax scale must be positive and finite");
-  if ((int64_t)S * 3 * H * kD * 2 > 0x7fffffffLL) fail("fusedMHA: one sequence of QKV must stay below 2 GiB");
+  if ((int64_t)S * 3 * H * D * 2 > 0x7fffffffLL) fail("fusedMHA: one sequence of QKV must stay below 2 GiB");
   // One 32-query block per wavefront: 64 queries per wavefront would halve the
   // LDS operand traffic per flop, but at 224 VGPRs only two wavefronts fit a
   // SIMD and the kernel measured slower at every shape tried.
   if (dt == DType::F16) {
-    launch<_Float16, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
+    if (D == 64) launch<_Float16, 64, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
+    else launch<_Float16, 128, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
   } else if (dt == DType::BF16) {
-    launch<bf16_t, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
+    if (D == 64) launch<bf16_t, 64, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
+    else launch<bf16_t, 128, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
   } else {
     fail("fusedMHA: element type must be fp16 or bf16");
   }

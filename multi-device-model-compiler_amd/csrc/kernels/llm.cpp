@@ -18,6 +18,8 @@
 // learned LayerNorm affine, optional key-padding lengths); the reference has
 // no such entry point.
 #include "common.hpp"
+
+#include <cmath>
 #include "mgpu_ops_internal.hpp"
 
 namespace mgpu {
@@ -76,8 +78,8 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
   if (!copyStream) fail("mgpuLLMDecodingContextLayer: gpuOpsInit() has not been called");
   if (batch < 0 || seq_len < 0 || d_model <= 0 || ffn <= 0 || heads <= 0)
     fail("mgpuLLMDecodingContextLayer: bad shape");
-  if (d_model % heads || d_model / heads != 64)
-    fail("mgpuLLMDecodingContextLayer: d_model / head_num must be 64");
+  if (d_model % heads || (d_model / heads != 64 && d_model / heads != 128))
+    fail("mgpuLLMDecodingContextLayer: d_model / head_num must be 64 or 128");
   if (batch == 0 || seq_len == 0) return;
   if (!input || !qkv || !gemm_weight || !gemm_bias || !ffn1_weight || !ffn1_bias || !ffn2_weight ||
       !ffn2_bias || !output)
@@ -120,7 +122,7 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
 
   // Attention context overwrites the first LayerNorm output, like the reference.
   fusedMHA(DType::F16, arena.at(oQkv), nullptr, arena.at(oLn), (int)batch, (int)seq_len,
-           (int)heads, 64, 0.125f, causal, stream);
+           (int)heads, (int)(d_model / heads), 1.0f / sqrtf((float)(d_model / heads)), causal, stream);
 
   castF32ToF16(arena.at(oWo), gemm_weight, d * d, copyStream);
   castF32ToF16(arena.at(oBo), gemm_bias, d, copyStream);
@@ -154,7 +156,7 @@ void bertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, cons
                          int64_t S, int64_t d, int64_t ffn, int64_t H, float eps,
                          hipStream_t stream) {
   if (B < 0 || S < 0 || d <= 0 || ffn <= 0 || H <= 0) fail("mgpuBertEncoderLayerF16: bad shape");
-  if (d % H || d / H != 64) fail("mgpuBertEncoderLayerF16: d_model / head_num must be 64");
+  if (d % H || (d / H != 64 && d / H != 128)) fail("mgpuBertEncoderLayerF16: d_model / head_num must be 64 or 128");
   if (B == 0 || S == 0) return;
   if (!x || !wqkv || !bqkv || !wo || !bo || !gamma1 || !beta1 || !w1 || !b1 || !w2 || !b2 ||
       !gamma2 || !beta2 || !out)
@@ -171,8 +173,8 @@ void bertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, cons
 
   matmulEx(DType::F16, x, wqkv, bqkv, arena.at(oQkv), nullptr, M, 3 * d, d, true, ACT_NONE, false,
            stream);
-  fusedMHA(DType::F16, arena.at(oQkv), seqlens, arena.at(oCtx), (int)B, (int)S, (int)H, 64, 0.125f,
-           false, stream);
+  fusedMHA(DType::F16, arena.at(oQkv), seqlens, arena.at(oCtx), (int)B, (int)S, (int)H, (int)(d / H),
+           1.0f / sqrtf((float)(d / H)), false, stream);
   matmulEx(DType::F16, arena.at(oCtx), wo, bo, arena.at(oProj), nullptr, M, d, d, true, ACT_NONE,
            false, stream);
   layerNorm(DType::F16, arena.at(oProj), x, gamma1, beta1, arena.at(oSum), arena.at(oH1), eps,

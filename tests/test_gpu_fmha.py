@@ -25,10 +25,10 @@ def run(pkg, gpu, qkv, lens=None, causal=False, scale=None):
     return pkg.fused_mha(to_dev(qkv, gpu), tl, scale=scale, causal=causal).cpu().numpy().astype(np.float32)
 
 
-def make_qkv(rng, B, S, H, std=1.0):
+def make_qkv(rng, B, S, H, std=1.0, D=64):
     # unit variance: logits ~ N(0, 1) at scale 1/8, outputs O(0.1 .. 1) - an error in
     # the softmax weights or a V tile paired with the wrong P is far above tolerance
-    return (rng.standard_normal((B, S, 3, H, 64)) * std).astype(np.float16)
+    return (rng.standard_normal((B, S, 3, H, D)) * std).astype(np.float16)
 
 
 def test_fmha_config2_b32_s128_h12(pkg, gpu, oracle):
@@ -102,6 +102,39 @@ def test_fmha_large_logits_and_other_scales(pkg, gpu, oracle, rng):
     qkv = make_qkv(rng, 1, 256, 1)
     qkv[0, :, 1, 0, :] *= np.linspace(0.05, 6.0, 256, dtype=np.float16)[:, None]
     assert excess(run(pkg, gpu, qkv, scale=1.0), oracle.fmha(qkv, scale=1.0), TOL_F16) <= 1.0
+
+
+@pytest.mark.parametrize("B,S,H,lens,causal", [
+    (2, 128, 8, None, False), (1, 1, 1, None, False), (2, 31, 2, None, False), (1, 32, 1, None, True),
+    (2, 33, 2, [33, 7], False), (1, 257, 3, None, True), (2, 512, 2, [512, 300], False), (3, 100, 2, [0, 1, 100], True),
+    (1, 1000, 1, [777], False),
+])
+def test_fmha_head_dim_128(pkg, gpu, oracle, rng, B, S, H, lens, causal):
+    """head_dim 128 (the reference's layer runs 8 heads of 128, LLM.cu:79-81 with
+    qkvToContext.cu:62-75): key tiles of 32, default scale 1/sqrt(128)."""
+    qkv = make_qkv(rng, B, S, H, D=128)
+    got = run(pkg, gpu, qkv, lens, causal=causal)
+    ref = oracle.fmha(qkv, lens, causal=causal)
+    assert got.shape == (B, S, H * 128)
+    assert excess(got, ref, TOL_F16) <= 1.0
+    dirty = qkv.copy()
+    if lens is not None:  # padding may hold anything
+        for b, l in enumerate(lens):
+            dirty[b, max(l, 0):, 1:] = np.float16(np.nan)
+        got = run(pkg, gpu, dirty, lens, causal=causal)
+        assert np.isfinite(got).all() and excess(got, ref, TOL_F16) <= 1.0
+
+
+def test_fmha_head_dim_128_bf16_and_peaked(pkg, gpu, oracle, rng):
+    import torch
+    f = rng.standard_normal((2, 200, 3, 2, 128)).astype(np.float32)
+    t = torch.from_numpy(f).to(gpu).to(torch.bfloat16)
+    got = pkg.fused_mha(t).float().cpu().numpy()
+    bits = t.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert excess(got, oracle.fmha(bits, bf16=True), TOL_BF16) <= 1.0
+    qkv = make_qkv(rng, 1, 320, 2, D=128)
+    for scale in (1.0 / np.sqrt(128), 0.5):  # 0.5: logits ~ N(0, 32), repeated overflow repair
+        assert excess(run(pkg, gpu, qkv, scale=scale), oracle.fmha(qkv, scale=scale), TOL_F16) <= 1.0, scale
 
 
 def test_fmha_padding_garbage_is_ignored(pkg, gpu, oracle, rng):

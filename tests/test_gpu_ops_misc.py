@@ -101,9 +101,10 @@ def test_bert_encoder_layer_config4(pkg, gpu, oracle):
         assert err.mean() <= 5e-4
 
 
-@pytest.mark.parametrize("causal,relu", [(True, True), (False, False)])
-def test_decoding_context_layer(pkg, gpu, oracle, rng, causal, relu):
-    B, S, d, ffn, H = 4, 128, 512, 2048, 8
+@pytest.mark.parametrize("causal,relu,d,H", [(True, True, 512, 8), (False, False, 512, 8), (True, True, 1024, 8)])
+def test_decoding_context_layer(pkg, gpu, oracle, rng, causal, relu, d, H):
+    """(1024, 8): the reference's own head geometry, 8 heads of 128."""
+    B, S, ffn = 4, 128, 2048
     f = lambda *s, sc=0.03: (sc * rng.standard_normal(s)).astype(np.float32)
     x = rng.standard_normal((B, S, d)).astype(np.float32)
     W = [f(d, 3 * d), f(d, d), f(d), f(d, ffn), f(ffn), f(ffn, d), f(d)]

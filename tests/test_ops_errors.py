@@ -20,7 +20,7 @@ def test_no_error_initially_and_query_clears(lib):
     take(lib)
     assert take(lib) is None
     lib.mgpuFusedMHAF16(1, None, 1, 1, 1, 1, 32, 0.125, 0, None)
-    assert "head_dim 64" in take(lib)
+    assert "head_dim must be 64 or 128" in take(lib)
     assert take(lib) is None
 
 
