@@ -114,6 +114,22 @@ void mgpuAddFusedQKVBiasTransposeF16(void *q_buf, void *k_buf, void *v_buf, void
  * (Ops.h:23-25; lib/Kernels/GPU/Ops.cu:57-120). */
 void mgpuMatmul(float *input, float *weight, float *bias, float *output, int64_t M, int64_t N,
                 int64_t K, mgpuStream_t stream);
+/* ---- convolution and pooling (NCHW fp32) ------------------------------- */
+/* output[N,OC,OH,OW] = act(conv(input[N,IC,H,W], weight[OC,IC,KH,KW]) + bias[OC] + postAdd),
+ * act = ReLU when hasContainRelu, identity otherwise; postAdd [N,OC,OH,OW] is
+ * read only when hasPostAdd.  Same argument list as the reference
+ * (Ops.h:27-33; lib/Kernels/GPU/Ops.cu:238-335).  OH / OW must follow from
+ * the other arguments; right / bottom padding is honoured. */
+void mgpuConv2d(float *input, float *weight, float *bias, float *output, float *postAdd, int64_t N,
+                int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t OH,
+                int64_t OW, int64_t PHL, int64_t PWL, int64_t PHR, int64_t PWR, int64_t SH, int64_t SW,
+                int64_t DH, int64_t DW, bool hasPostAdd, bool hasContainRelu, mgpuStream_t stream);
+/* output[N,C,OH,OW] = window maximum (method 0, padding ignored) or window
+ * mean counting the padding as zeros (method 1) (Ops.h:35-41; Ops.cu:337-374). */
+void mgpuPool2d(float *input, float *output, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH,
+                int64_t OW, int64_t KH, int64_t KW, int64_t PHL, int64_t PWL, int64_t PHR, int64_t PWR,
+                int64_t SH, int64_t SW, int64_t method, mgpuStream_t stream);
+
 /* output = act(input . weight + bias) + residual; replaces mgpuMatmulEx<T>
  * (Ops.h:51-55; Ops.cu:134-234).  hasRelu: 0 none, 1 ReLU; hasRelu == 2 selects
  * GELU (erf form), which the reference does not have.  fp32 accumulation. */

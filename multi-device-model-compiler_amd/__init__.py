@@ -60,6 +60,8 @@ OPS_SIGNATURES = {
     "mgpuCastF16ToF32": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
     "mgpuAddFusedQKVBiasTransposeF16": (None, [_c_void_p] * 5 + [_c_int32] * 5 + [_c_void_p]),
     "mgpuMatmul": (None, [_c_void_p] * 4 + [_c_int64] * 3 + [_c_void_p]),
+    "mgpuConv2d": (None, [_c_void_p] * 5 + [_c_int64] * 17 + [ctypes.c_bool] * 2 + [_c_void_p]),
+    "mgpuPool2d": (None, [_c_void_p] * 2 + [_c_int64] * 15 + [_c_void_p]),
     "mgpuMatmulExF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuMatmulExF32": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuLLMDecodingContextLayer": (None, [_c_void_p] * 9 + [_c_int64] * 5 + [ctypes.c_bool] * 3 + [_c_void_p]),
@@ -269,6 +271,41 @@ def matmul_ex(x, w, bias=None, residual=None, act: int = ACT_NONE, stream=None):
     fn = lib.mgpuMatmulExF16 if x.dtype == torch.float16 else lib.mgpuMatmulExF32
     fn(_ptr(x), _ptr(w), _ptr(bias), _ptr(out), _ptr(residual), M, N, K,
        1 if bias is not None else 0, act, 1 if residual is not None else 0, _stream_handle(stream))
+    _check(lib)
+    return out
+
+
+def _conv_out(size, k, pl, pr, s, d=1):
+    return (size + pl + pr - d * (k - 1) - 1) // s + 1
+
+
+def conv2d(x, w, bias, post_add=None, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), relu=False, stream=None):
+    """NCHW fp32; pad = (top, left, bottom, right)."""
+    import torch
+    N, IC, H, W = x.shape
+    OC, IC2, KH, KW = w.shape
+    assert IC == IC2
+    OH = _conv_out(H, KH, pad[0], pad[2], stride[0], dilation[0])
+    OW = _conv_out(W, KW, pad[1], pad[3], stride[1], dilation[1])
+    out = torch.empty((N, OC, OH, OW), dtype=x.dtype, device=x.device)
+    lib = ops()
+    lib.mgpuConv2d(_ptr(x), _ptr(w), _ptr(bias), _ptr(out), _ptr(post_add), N, IC, H, W, OC, KH, KW, OH, OW,
+                   pad[0], pad[1], pad[2], pad[3], stride[0], stride[1], dilation[0], dilation[1],
+                   post_add is not None, relu, _stream_handle(stream))
+    _check(lib)
+    return out
+
+
+def pool2d(x, kernel, pad=(0, 0, 0, 0), stride=(1, 1), method="max", stream=None):
+    """NCHW fp32; method "max" or "avg" (average counts the padding)."""
+    import torch
+    N, C, H, W = x.shape
+    OH = _conv_out(H, kernel[0], pad[0], pad[2], stride[0])
+    OW = _conv_out(W, kernel[1], pad[1], pad[3], stride[1])
+    out = torch.empty((N, C, OH, OW), dtype=x.dtype, device=x.device)
+    lib = ops()
+    lib.mgpuPool2d(_ptr(x), _ptr(out), N, C, H, W, OH, OW, kernel[0], kernel[1], pad[0], pad[1], pad[2], pad[3],
+                   stride[0], stride[1], 0 if method == "max" else 1, _stream_handle(stream))
     _check(lib)
     return out
 

@@ -171,6 +171,36 @@ bool emitOp(Lowering &L, const DeviceOp &op, std::string &error) {
                        i32(actCode), i32(op.operands[3] >= 0)}));
     return true;
   }
+  if (n == "device.conv2d" || n == "device.pool2d") {
+    auto ints = [&](const char *key, std::vector<int64_t> fallback) {
+      auto a = op.attrs.find(key);
+      return a == op.attrs.end() ? fallback : a->second.ints;
+    };
+    const TensorType &x = inT(0), &y = plan.values[op.results[0]].type;
+    const std::vector<int64_t> pad = ints("pad", {0, 0, 0, 0}), stride = ints("stride", {1, 1});
+    std::vector<CallArg> args;
+    if (n == "device.conv2d") {
+      // argument order of ConvertDeviceToLLVM.cpp:533-548: pointers, N IC H W OC KH KW OH OW,
+      // PHL PWL PHR PWR SH SW DH DW, hasPostAdd, containRelu
+      const TensorType &w = inT(1);
+      const std::vector<int64_t> dil = ints("dilation", {1, 1});
+      args = {in(0), in(1), in(2), out(0), in(3)};
+      for (int64_t v : {x.shape[0], x.shape[1], x.shape[2], x.shape[3], w.shape[0], w.shape[2], w.shape[3], y.shape[2],
+                        y.shape[3], pad[0], pad[1], pad[2], pad[3], stride[0], stride[1], dil[0], dil[1]})
+        args.push_back(i64(v));
+      args.push_back(boolean(op.operands[3] >= 0));
+      args.push_back(boolean(attrBool(op, "containRelu", false)));
+      L.call(gpu ? "mgpuConv2d" : "mcpuConv2d", withStream(args));
+    } else {
+      const std::vector<int64_t> k = ints("kernel", {1, 1});
+      args = {in(0), out(0)};
+      for (int64_t v : {x.shape[0], x.shape[1], x.shape[2], x.shape[3], y.shape[2], y.shape[3], k[0], k[1], pad[0], pad[1],
+                        pad[2], pad[3], stride[0], stride[1], (int64_t)(attrString(op, "method", "max") == "avg")})
+        args.push_back(i64(v));
+      L.call(gpu ? "mgpuPool2d" : "mcpuPool2d", withStream(args));
+    }
+    return true;
+  }
   if (n == "device.cast") {
     if (!gpu) return noCpu();
     L.call(inT(0).elem == ElemType::F32 ? "mgpuCastF32ToF16" : "mgpuCastF16ToF32",

@@ -460,6 +460,59 @@ bool verifyOp(const DevicePlan &plan, const DeviceOp &op, std::string &error) {
     }
     return true;
   }
+  if (n == "device.conv2d") { // Conv2DOp::verify, DeviceDialect.cpp:114-140, plus the size arithmetic
+    if (!v.counts(4, 1) || !v.required({0, 1, 2}) ||
+        !v.attrKinds({{"pad", AttrValue::IntList}, {"stride", AttrValue::IntList}, {"dilation", AttrValue::IntList},
+                      {"kernel", AttrValue::IntList}, {"containRelu", AttrValue::Bool}})) return false;
+    const TensorType &x = v.in(0), &w = v.in(1), &y = v.out(0);
+    if (x.elem != ElemType::F32 || w.elem != ElemType::F32 || y.elem != ElemType::F32) return v.fail("built for f32");
+    if (x.shape.size() != 4 || w.shape.size() != 4 || y.shape.size() != 4) return v.fail("input, weight and output are rank 4 (NCHW / OIHW)");
+    if (x.shape[0] != y.shape[0] || x.shape[1] != w.shape[1] || y.shape[1] != w.shape[0])
+      return v.fail("batch or channel counts of input, weight and output disagree");
+    if (!v.vectorOf(2, w.shape[0], ElemType::F32, "bias")) return false;
+    if (v.present(3) && v.in(3) != y) return v.fail("postadd has the type of the output");
+    std::vector<int64_t> pad{0, 0, 0, 0}, stride{1, 1}, dil{1, 1};
+    const std::pair<const char *, std::vector<int64_t> *> lists[] = {{"pad", &pad}, {"stride", &stride}, {"dilation", &dil}};
+    for (const auto &kv : lists) {
+      auto a = op.attrs.find(kv.first);
+      if (a == op.attrs.end()) continue;
+      if (a->second.ints.size() != kv.second->size()) return v.fail(std::string(kv.first) + " has the wrong number of entries");
+      *kv.second = a->second.ints;
+    }
+    auto k = op.attrs.find("kernel");
+    if (k != op.attrs.end() && k->second.ints != std::vector<int64_t>{w.shape[2], w.shape[3]}) return v.fail("kernel disagrees with the weight shape");
+    for (int d = 0; d < 2; d++) {
+      if (stride[d] <= 0 || dil[d] <= 0 || pad[d] < 0 || pad[d + 2] < 0) return v.fail("bad pad, stride or dilation");
+      const int64_t span = x.shape[2 + d] + pad[d] + pad[d + 2] - dil[d] * (w.shape[2 + d] - 1) - 1;
+      if (span < 0 || y.shape[2 + d] != span / stride[d] + 1) return v.fail("output size does not follow from input, kernel, pad, stride and dilation");
+    }
+    return true;
+  }
+  if (n == "device.pool2d") {
+    if (!v.counts(1, 1) || !v.required({0}) ||
+        !v.attrKinds({{"kernel", AttrValue::IntList}, {"pad", AttrValue::IntList}, {"stride", AttrValue::IntList},
+                      {"method", AttrValue::String}})) return false;
+    const TensorType &x = v.in(0), &y = v.out(0);
+    if (x.elem != ElemType::F32 || y.elem != ElemType::F32) return v.fail("built for f32");
+    if (x.shape.size() != 4 || y.shape.size() != 4 || x.shape[0] != y.shape[0] || x.shape[1] != y.shape[1])
+      return v.fail("input and output are NCHW with the same batch and channel counts");
+    auto k = op.attrs.find("kernel");
+    if (k == op.attrs.end() || k->second.ints.size() != 2) return v.fail("needs kernel = [KH, KW]");
+    std::vector<int64_t> pad{0, 0, 0, 0}, stride{1, 1};
+    auto p = op.attrs.find("pad");
+    if (p != op.attrs.end()) { if (p->second.ints.size() != 4) return v.fail("pad has four entries"); pad = p->second.ints; }
+    auto st = op.attrs.find("stride");
+    if (st != op.attrs.end()) { if (st->second.ints.size() != 2) return v.fail("stride has two entries"); stride = st->second.ints; }
+    auto m = op.attrs.find("method");
+    if (m == op.attrs.end() || (m->second.text != "max" && m->second.text != "avg")) return v.fail("method is \"max\" or \"avg\"");
+    for (int d = 0; d < 2; d++) {
+      const int64_t kk = k->second.ints[d];
+      if (kk <= 0 || stride[d] <= 0 || pad[d] < 0 || pad[d + 2] < 0 || pad[d] >= kk || pad[d + 2] >= kk) return v.fail("bad kernel, pad or stride");
+      const int64_t span = x.shape[2 + d] + pad[d] + pad[d + 2] - kk;
+      if (span < 0 || y.shape[2 + d] != span / stride[d] + 1) return v.fail("output size does not follow from input, kernel, pad and stride");
+    }
+    return true;
+  }
   if (n == "device.reshape") { // a view: same buffer, another shape (memref.reshape)
     if (!v.counts(1, 1) || !v.required({0}) || !v.attrKinds({})) return false;
     if (v.in(0).elem != v.out(0).elem || v.in(0).numel() != v.out(0).numel())

@@ -114,6 +114,26 @@ bool dispatch(Machine &m, const RuntimeCall &c) {
     return true;
   }
   if (n == "mgpuCastF32ToF16" || n == "mgpuCastF16ToF32") { ((void (*)(P, P, size_t, P))fn)(p(0), p(1), (size_t)l(2), p(3)); return true; }
+  if (n == "mgpuConv2d" || n == "mcpuConv2d") {
+    typedef void (*Gpu)(P, P, P, P, P, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, bool, bool, P);
+    typedef void (*Cpu)(P, P, P, P, P, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, bool, bool);
+    if (n[1] == 'g')
+      ((Gpu)fn)(p(0), p(1), p(2), p(3), p(4), l(5), l(6), l(7), l(8), l(9), l(10), l(11), l(12), l(13), l(14), l(15), l(16),
+                l(17), l(18), l(19), l(20), l(21), b(22), b(23), p(24));
+    else
+      ((Cpu)fn)(p(0), p(1), p(2), p(3), p(4), l(5), l(6), l(7), l(8), l(9), l(10), l(11), l(12), l(13), l(14), l(15), l(16),
+                l(17), l(18), l(19), l(20), l(21), b(22), b(23));
+    return true;
+  }
+  if (n == "mgpuPool2d" || n == "mcpuPool2d") {
+    typedef void (*Gpu)(P, P, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, P);
+    typedef void (*Cpu)(P, P, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L);
+    if (n[1] == 'g')
+      ((Gpu)fn)(p(0), p(1), l(2), l(3), l(4), l(5), l(6), l(7), l(8), l(9), l(10), l(11), l(12), l(13), l(14), l(15), l(16), p(17));
+    else
+      ((Cpu)fn)(p(0), p(1), l(2), l(3), l(4), l(5), l(6), l(7), l(8), l(9), l(10), l(11), l(12), l(13), l(14), l(15), l(16));
+    return true;
+  }
   if (n == "mgpuMatmul") { ((void (*)(P, P, P, P, L, L, L, P))fn)(p(0), p(1), p(2), p(3), l(4), l(5), l(6), p(7)); return true; }
   if (n == "mgpuMatmulExF16" || n == "mgpuMatmulExF32") {
     ((void (*)(P, P, P, P, P, L, L, L, I, I, I, P))fn)(p(0), p(1), p(2), p(3), p(4), l(5), l(6), l(7), i(8), i(9), i(10), p(11));

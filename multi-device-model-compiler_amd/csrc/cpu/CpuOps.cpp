@@ -82,6 +82,69 @@ void mcpuMatmul(float *input, float *weight, float *bias, float *output, int64_t
   }
 }
 
+// NCHW fp32 convolution (cross-correlation) + bias + optional postAdd + optional
+// ReLU; the CPU side of mgpuConv2d (reference: oneDNN convolution_forward with
+// post-ops, lib/Kernels/CPU/Ops.cpp; Ops.h:24-29).  One output row at a time,
+// the tap loop outermost so that the inner loop runs along the row.
+void mcpuConv2d(float *input, float *weight, float *bias, float *output, float *postAdd, int64_t N,
+                int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t OH,
+                int64_t OW, int64_t PHL, int64_t PWL, int64_t /*PHR*/, int64_t /*PWR*/, int64_t SH,
+                int64_t SW, int64_t DH, int64_t DW, bool hasPostAdd, bool hasContainRelu) {
+#pragma omp parallel for collapse(3) schedule(static)
+  for (int64_t n = 0; n < N; n++)
+    for (int64_t oc = 0; oc < OC; oc++)
+      for (int64_t oh = 0; oh < OH; oh++) {
+        float *row = output + ((n * OC + oc) * OH + oh) * OW;
+        for (int64_t ow = 0; ow < OW; ow++) row[ow] = bias[oc];
+        for (int64_t ic = 0; ic < IC; ic++)
+          for (int64_t kh = 0; kh < KH; kh++) {
+            const int64_t ih = oh * SH - PHL + kh * DH;
+            if (ih < 0 || ih >= H) continue;
+            const float *src = input + ((n * IC + ic) * H + ih) * W;
+            for (int64_t kw = 0; kw < KW; kw++) {
+              const float wv = weight[((oc * IC + ic) * KH + kh) * KW + kw];
+              const int64_t off = kw * DW - PWL;
+              // ow range with 0 <= ow*SW + off < W
+              int64_t lo = off < 0 ? (-off + SW - 1) / SW : 0;
+              int64_t hi = (W - 1 - off) >= 0 ? (W - 1 - off) / SW + 1 : 0;
+              if (hi > OW) hi = OW;
+#pragma omp simd
+              for (int64_t ow = lo; ow < hi; ow++) row[ow] += wv * src[ow * SW + off];
+            }
+          }
+        if (hasPostAdd) {
+          const float *add = postAdd + ((n * OC + oc) * OH + oh) * OW;
+          for (int64_t ow = 0; ow < OW; ow++) row[ow] += add[ow];
+        }
+        if (hasContainRelu)
+          for (int64_t ow = 0; ow < OW; ow++) row[ow] = row[ow] > 0.0f ? row[ow] : 0.0f;
+      }
+}
+
+// method 0: window maximum over the taps inside the image; 1: window sum over
+// those taps divided by KH*KW (Ops.h:31-36).
+void mcpuPool2d(float *input, float *output, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH,
+                int64_t OW, int64_t KH, int64_t KW, int64_t PHL, int64_t PWL, int64_t /*PHR*/,
+                int64_t /*PWR*/, int64_t SH, int64_t SW, int64_t method) {
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t pl = 0; pl < N * C; pl++)
+    for (int64_t oh = 0; oh < OH; oh++)
+      for (int64_t ow = 0; ow < OW; ow++) {
+        float acc = method ? 0.0f : -INFINITY;
+        for (int64_t kh = 0; kh < KH; kh++) {
+          const int64_t ih = oh * SH - PHL + kh;
+          if (ih < 0 || ih >= H) continue;
+          for (int64_t kw = 0; kw < KW; kw++) {
+            const int64_t iw = ow * SW - PWL + kw;
+            if (iw < 0 || iw >= W) continue;
+            const float v = input[(pl * H + ih) * W + iw];
+            acc = method ? acc + v : (v > acc ? v : acc);
+          }
+        }
+        output[(pl * OH + oh) * OW + ow] = method ? acc / (float)(KH * KW) : acc;
+      }
+}
+
 void mcpuAddF32(const float *a, const float *b, float *c, int64_t n) {
 #pragma omp parallel for schedule(static)
   for (int64_t i = 0; i < n; i++) c[i] = a[i] + b[i];

@@ -234,6 +234,22 @@ void mgpuMatmul(float *input, float *weight, float *bias, float *output, int64_t
                    mgpu::ACT_NONE, false, S(stream));
   });
 }
+void mgpuConv2d(float *input, float *weight, float *bias, float *output, float *postAdd, int64_t N,
+                int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t OH,
+                int64_t OW, int64_t PHL, int64_t PWL, int64_t PHR, int64_t PWR, int64_t SH, int64_t SW,
+                int64_t DH, int64_t DW, bool hasPostAdd, bool hasContainRelu, mgpuStream_t stream) {
+  guarded([&] {
+    mgpu::conv2d(input, weight, bias, output, postAdd, N, IC, H, W, OC, KH, KW, OH, OW, PHL, PWL, PHR, PWR,
+                 SH, SW, DH, DW, hasPostAdd, hasContainRelu, S(stream));
+  });
+}
+void mgpuPool2d(float *input, float *output, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH,
+                int64_t OW, int64_t KH, int64_t KW, int64_t PHL, int64_t PWL, int64_t PHR, int64_t PWR,
+                int64_t SH, int64_t SW, int64_t method, mgpuStream_t stream) {
+  guarded([&] {
+    mgpu::pool2d(input, output, N, C, H, W, OH, OW, KH, KW, PHL, PWL, PHR, PWR, SH, SW, method, S(stream));
+  });
+}
 void mgpuMatmulExF16(void *input, void *weight, void *bias, void *output, void *residual,
                      int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
                      int32_t hasResidual, mgpuStream_t stream) {

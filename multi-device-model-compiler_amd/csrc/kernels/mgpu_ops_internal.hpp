@@ -37,6 +37,14 @@ void matmulEx(DType dt, const void *input, const void *weight, const void *bias,
               const void *residual, int64_t M, int64_t N, int64_t K, bool hasBias, int act,
               bool hasResidual, hipStream_t stream);
 
+void conv2d(const float *input, const float *weight, const float *bias, float *output, const float *postAdd,
+            int64_t N, int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t OH,
+            int64_t OW, int64_t PHL, int64_t PWL, int64_t PHR, int64_t PWR, int64_t SH, int64_t SW, int64_t DH,
+            int64_t DW, bool hasPostAdd, bool relu, hipStream_t stream);
+void pool2d(const float *input, float *output, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW,
+            int64_t KH, int64_t KW, int64_t PHL, int64_t PWL, int64_t PHR, int64_t PWR, int64_t SH, int64_t SW,
+            int64_t method, hipStream_t stream);
+
 void llmInit();
 void llmDeinit();
 void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *gemm_bias,

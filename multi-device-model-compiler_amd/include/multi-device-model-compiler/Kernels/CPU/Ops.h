@@ -17,6 +17,13 @@ extern "C" {
 void mcpuMatmul(float *input, float *weight, float *bias, float *output, int64_t M, int64_t N,
                 int64_t K);
 // CPU twins of the GPU entry points of mgpu_ops.h that have no reference name.
+void mcpuConv2d(float *input, float *weight, float *bias, float *output, float *postAdd, int64_t N,
+                int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t OH,
+                int64_t OW, int64_t PHL, int64_t PWL, int64_t PHR, int64_t PWR, int64_t SH, int64_t SW,
+                int64_t DH, int64_t DW, bool hasPostAdd, bool hasContainRelu);
+void mcpuPool2d(float *input, float *output, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH,
+                int64_t OW, int64_t KH, int64_t KW, int64_t PHL, int64_t PWL, int64_t PHR, int64_t PWR,
+                int64_t SH, int64_t SW, int64_t method /* 0 - max, 1 - avg */);
 void mcpuAddF32(const float *a, const float *b, float *c, int64_t n);
 void mcpuLayerNormF32(const float *input, const float *gamma, const float *beta, float *output,
                       float eps, int32_t m, int32_t n);

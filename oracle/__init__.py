@@ -257,3 +257,37 @@ def ref_add_3x640x640(a, b):
                                 shape=(3, 640, 640)).copy()
     libc.free(out.allocated)
     return res
+
+
+def _out_size(size, k, pl, pr, s, d=1):
+    return (size + pl + pr - d * (k - 1) - 1) // s + 1
+
+
+def conv2d(x, w, bias, post_add=None, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), relu=False):
+    """NCHW fp32 cross-correlation + bias (+ post_add) (+ ReLU); pad = (top, left, bottom, right)."""
+    x, w, bias, post_add = _c(x, np.float32), _c(w, np.float32), _c(bias, np.float32), _c(post_add, np.float32)
+    N, IC, H, W = x.shape
+    OC, IC2, KH, KW = w.shape
+    assert IC == IC2 and bias.shape == (OC,)
+    OH = _out_size(H, KH, pad[0], pad[2], stride[0], dilation[0])
+    OW = _out_size(W, KW, pad[1], pad[3], stride[1], dilation[1])
+    y = np.empty((N, OC, OH, OW), np.float32)
+    i64 = ctypes.c_int64
+    lib().oracle_conv2d(_p(x), _p(w), _p(bias), _p(post_add), _p(y), *[i64(v) for v in (
+        N, IC, H, W, OC, KH, KW, OH, OW, pad[0], pad[1], stride[0], stride[1], dilation[0], dilation[1])],
+        ctypes.c_int(1 if relu else 0))
+    return y
+
+
+def pool2d(x, kernel, pad=(0, 0, 0, 0), stride=(1, 1), method="max"):
+    """NCHW fp32; "max" ignores the padding, "avg" divides by the full window."""
+    x = _c(x, np.float32)
+    N, C, H, W = x.shape
+    OH = _out_size(H, kernel[0], pad[0], pad[2], stride[0])
+    OW = _out_size(W, kernel[1], pad[1], pad[3], stride[1])
+    y = np.empty((N, C, OH, OW), np.float32)
+    i64 = ctypes.c_int64
+    lib().oracle_pool2d(_p(x), _p(y), *[i64(v) for v in (
+        N * C, H, W, OH, OW, kernel[0], kernel[1], pad[0], pad[1], stride[0], stride[1])],
+        ctypes.c_int(0 if method == "max" else 1))
+    return y

@@ -527,3 +527,65 @@ ORACLE_API void oracle_bert_layer_f16(const uint16_t *x, const uint16_t *wqkv, c
   free(t0); free(t1); free(t2); free(sum); free(qkv_h); free(ctx_h); free(pr_h); free(h1_h);
   free(f_h); free(o_h);
 }
+
+/* ---- convolution and pooling, NCHW fp32 --------------------------------
+ * y[n,oc,oh,ow] = act(sum_{ic,kh,kw} x[n,ic,oh*SH-PHL+kh*DH,ow*SW-PWL+kw*DW] * w[oc,ic,kh,kw]
+ *                     + bias[oc] + add[n,oc,oh,ow])
+ * with taps outside the image reading zero, i.e. cross-correlation, the form of
+ * ONNX Conv, of torch conv2d and of the reference's CPU path (oneDNN
+ * convolution_forward, lib/Kernels/CPU/Ops.cpp).  The reference's GPU entry
+ * point sets CUDNN_CONVOLUTION (lib/Kernels/GPU/Ops.cu:251-253), which cuDNN
+ * defines with the filter flipped; the CPU path is the parity standard, so the
+ * un-flipped form is restated here and pinned against torch.nn.functional.conv2d.
+ * Accumulation in double.  relu: max(v, 0) with NaN -> 0
+ * (CUDNN_NOT_PROPAGATE_NAN, Ops.cu:289-293). */
+ORACLE_API void oracle_conv2d(const float *x, const float *w, const float *bias, const float *add, float *y, int64_t N,
+                   int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t OH, int64_t OW,
+                   int64_t PHL, int64_t PWL, int64_t SH, int64_t SW, int64_t DH, int64_t DW, int relu) {
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t n = 0; n < N; n++)
+    for (int64_t oc = 0; oc < OC; oc++)
+      for (int64_t oh = 0; oh < OH; oh++)
+        for (int64_t ow = 0; ow < OW; ow++) {
+          double acc = 0.0;
+          for (int64_t ic = 0; ic < IC; ic++)
+            for (int64_t kh = 0; kh < KH; kh++) {
+              const int64_t ih = oh * SH - PHL + kh * DH;
+              if (ih < 0 || ih >= H) continue;
+              for (int64_t kw = 0; kw < KW; kw++) {
+                const int64_t iw = ow * SW - PWL + kw * DW;
+                if (iw < 0 || iw >= W) continue;
+                acc += (double)x[((n * IC + ic) * H + ih) * W + iw] * (double)w[((oc * IC + ic) * KH + kh) * KW + kw];
+              }
+            }
+          const int64_t o = ((n * OC + oc) * OH + oh) * OW + ow;
+          double v = acc + (double)bias[oc] + (add ? (double)add[o] : 0.0);
+          if (relu) v = v > 0.0 ? v : 0.0; /* NaN compares false: 0 */
+          y[o] = (float)v;
+        }
+}
+
+/* method 0: maximum over the taps inside the image (padding ignored, NaN taps
+ * ignored: CUDNN_NOT_PROPAGATE_NAN); method 1: sum of the taps inside the image
+ * divided by KH*KW (CUDNN_POOLING_AVERAGE_COUNT_INCLUDE_PADDING, Ops.cu:345-351). */
+ORACLE_API void oracle_pool2d(const float *x, float *y, int64_t planes, int64_t H, int64_t W, int64_t OH, int64_t OW,
+                   int64_t KH, int64_t KW, int64_t PHL, int64_t PWL, int64_t SH, int64_t SW, int method) {
+#pragma omp parallel for schedule(static)
+  for (int64_t pl = 0; pl < planes; pl++)
+    for (int64_t oh = 0; oh < OH; oh++)
+      for (int64_t ow = 0; ow < OW; ow++) {
+        double acc = method ? 0.0 : -INFINITY;
+        for (int64_t kh = 0; kh < KH; kh++) {
+          const int64_t ih = oh * SH - PHL + kh;
+          if (ih < 0 || ih >= H) continue;
+          for (int64_t kw = 0; kw < KW; kw++) {
+            const int64_t iw = ow * SW - PWL + kw;
+            if (iw < 0 || iw >= W) continue;
+            const double v = x[(pl * H + ih) * W + iw];
+            if (method) acc += v;
+            else if (v > acc) acc = v;
+          }
+        }
+        y[(pl * OH + oh) * OW + ow] = (float)(method ? acc / (double)(KH * KW) : acc);
+      }
+}

@@ -116,6 +116,21 @@ def test_bert_layer_plan_keeps_values_on_the_device_and_views_share_a_buffer():
     assert "4096, 3072, 768, 1 : i32, 2 : i32, 0 : i32, %KernelStream)" in out
 
 
+def test_conv_and_pool_lower_with_the_reference_argument_order():
+    """ConvertDeviceToLLVM.cpp:533-548,612-627: pointers, then N IC H W OC KH KW OH OW, PHL PWL PHR PWR,
+    SH SW, DH DW, hasPostAdd, containRelu, stream; pool: N C H W OH OW KH KW PHL PWL PHR PWR SH SW method."""
+    r = lower(os.path.join(PLANS, "resnet_block.plan"))
+    assert r.returncode == 0, r.stderr
+    assert ("mgpuConv2d(%d0, %d1, %d2, %d3, null, 4, 64, 28, 28, 64, 3, 3, 28, 28, 1, 1, 1, 1, 1, 1, 1, 1, "
+            "false, true, %KernelStream)") in r.stdout
+    assert ("mgpuConv2d(%d3, %d4, %d5, %d6, %d0, 4, 64, 28, 28, 64, 3, 3, 28, 28, 1, 1, 1, 1, 1, 1, 1, 1, "
+            "true, true, %KernelStream)") in r.stdout
+    assert "mgpuPool2d(%d6, %d7, 4, 64, 28, 28, 14, 14, 2, 2, 0, 0, 0, 0, 2, 2, 0, %KernelStream)" in r.stdout
+    # the shortcut keeps %x on the device until the second convolution has read it
+    lines = r.stdout.splitlines()
+    assert lines.index("mgpuMemFree(%d0, %DataStream)") > [i for i, l in enumerate(lines) if "mgpuConv2d" in l][1]
+
+
 def test_plan_round_trip(tmp_path):
     src = os.path.join(PLANS, "bert_layer.plan")
     printed = lower(src, "--emit", "plan")
@@ -230,6 +245,41 @@ def test_cpu_runner_executes_plans(tmp_path, oracle, rng):
     o, _ = run_cpu_plan(tmp_path, text, [qkv, lens], np.float16, (2, 70, 128))
     ref = oracle.fmha(qkv, lens, causal=True)
     assert np.abs(o.astype(np.float32) - ref).max() <= 2e-3 * max(1.0, np.abs(ref).max())
+
+
+def test_cpu_runner_executes_the_resnet_block(tmp_path, oracle, rng):
+    text = open(os.path.join(PLANS, "resnet_block.plan")).read().replace(" 4x64x", " 2x64x")
+    c = 64
+    w1, w2 = [(rng.standard_normal((c, c, 3, 3)) / 24).astype(np.float32) for _ in range(2)]
+    b1, b2 = [rng.standard_normal(c).astype(np.float32) for _ in range(2)]
+    for name, a in (("w1", w1), ("b1", b1), ("w2", w2), ("b2", b2)):
+        a.tofile(str(tmp_path / f"{name}.dat"))
+    x = rng.standard_normal((2, c, 28, 28)).astype(np.float32)
+    y, _ = run_cpu_plan(tmp_path, text, [x], np.float32, (2, c, 14, 14))
+    h = oracle.conv2d(x, w1, b1, None, (1, 1, 1, 1), relu=True)
+    r = oracle.conv2d(h, w2, b2, x, (1, 1, 1, 1), relu=True)
+    ref = oracle.pool2d(r, (2, 2), stride=(2, 2))
+    assert np.abs(y - ref).max() <= 1e-4
+
+
+def test_conv_pool_verifier_messages(tmp_path):
+    head = "func @f(%x: 1x2x8x8xf32, %w: 3x2x3x3xf32, %b: 3xf32) -> (%y: 1x3x8x8xf32) {\n"
+    for body, message in [
+        ("  %y = device.conv2d %x, %w, %b, none {pad = [1, 1, 1, 1]} : 1x3x8x8xf32\n  return\n}\n", None),
+        ("  %y = device.conv2d %x, %w, %b, none : 1x3x8x8xf32\n  return\n}\n", "output size does not follow"),
+        ("  %y = device.conv2d %x, %w, %x, none {pad = [1, 1, 1, 1]} : 1x3x8x8xf32\n  return\n}\n", "bias must be 3xf32"),
+        ("  %y = device.conv2d %x, %w, %b, none {pad = [1, 1, 1, 1], kernel = [5, 5]} : 1x3x8x8xf32\n  return\n}\n",
+         "kernel disagrees"),
+        ("  %y = device.conv2d %w, %w, %b, none {pad = [1, 1, 1, 1]} : 1x3x8x8xf32\n  return\n}\n", "batch or channel counts"),
+        ("  %t = device.pool2d %x {kernel = [2, 2], stride = [2, 2], method = \"min\"} : 1x2x4x4xf32\n  return\n}\n", "method is"),
+        ("  %t = device.pool2d %x {kernel = [2, 2], stride = [2, 2], method = \"avg\"} : 1x2x5x4xf32\n  return\n}\n",
+         "output size does not follow"),
+    ]:
+        r = lower_text(tmp_path, head + body)
+        if message is None:
+            assert r.returncode == 0, r.stderr
+        else:
+            assert r.returncode == 1 and message in r.stderr, (message, r.stderr)
 
 
 def test_cpu_runner_reports_missing_lowerings_and_bad_files(tmp_path):

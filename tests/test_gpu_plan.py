@@ -106,3 +106,22 @@ def test_multi_head_attention_layer_op(pkg, gpu, tmp_path, oracle):
     got, _ = run_plan(pkg, plan, [x] + W, np.float32, (B, S, d), tmp_path)
     ref = oracle.decoding_context_layer(x, *W, heads=H, causal=True, act=oracle.ACT_RELU)
     assert np.all(np.abs(got - ref) <= layer_tol(ref))
+
+
+def test_resnet_block_plan(pkg, gpu, tmp_path, oracle):
+    """conv + ReLU, conv + shortcut + ReLU, max pool: device.conv2d / device.pool2d through
+    mgpuConv2d / mgpuPool2d, the shortcut operand staying on the device across two ops."""
+    rng = np.random.Generator(np.random.PCG64(79))
+    c = 64
+    plan = tmp_path / "resnet_block.plan"
+    plan.write_text(open(os.path.join(PLANS, "resnet_block.plan")).read())
+    w1, w2 = [(rng.standard_normal((c, c, 3, 3)) / 24).astype(np.float32) for _ in range(2)]
+    b1, b2 = [rng.standard_normal(c).astype(np.float32) for _ in range(2)]
+    for name, a in (("w1", w1), ("b1", b1), ("w2", w2), ("b2", b2)):
+        a.tofile(str(tmp_path / f"{name}.dat"))
+    x = rng.standard_normal((4, c, 28, 28)).astype(np.float32)
+    y, _ = run_plan(pkg, plan, [x], np.float32, (4, c, 14, 14), tmp_path)
+    h = oracle.conv2d(x, w1, b1, None, (1, 1, 1, 1), relu=True)
+    r = oracle.conv2d(h, w2, b2, x, (1, 1, 1, 1), relu=True)
+    ref = oracle.pool2d(r, (2, 2), stride=(2, 2))
+    assert np.all(np.abs(y - ref) <= 4e-3 * (1.0 + np.abs(ref)))
