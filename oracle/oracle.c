@@ -2,7 +2,8 @@
  * CPU oracle for the device kernel library: TEST INFRASTRUCTURE ONLY.
  *
  * This file restates, in plain C, what the reference computes on the path
- *   add -> LayerNorm -> fused multi-head attention -> encoder layer.
+ *   add -> LayerNorm -> fused multi-head attention -> encoder layer,
+ * plus the convolution / pooling entry points of the same library.
  * It is the checker that the HIP kernels are compared with and the CPU
  * baseline that bench.py times; the product library never links or calls it.
  *
@@ -538,7 +539,10 @@ ORACLE_API void oracle_bert_layer_f16(const uint16_t *x, const uint16_t *wqkv, c
  * defines with the filter flipped; the CPU path is the parity standard, so the
  * un-flipped form is restated here and pinned against torch.nn.functional.conv2d.
  * Accumulation in double.  relu: max(v, 0) with NaN -> 0
- * (CUDNN_NOT_PROPAGATE_NAN, Ops.cu:289-293). */
+ * (CUDNN_NOT_PROPAGATE_NAN, Ops.cu:289-293).
+ * Pinned by tests/test_oracle_conv_pool.py: torch CPU conv2d in fp64 over
+ * padding / stride / dilation cases, hand-computed cases (filter orientation,
+ * bias, ReLU, postAdd, border counts), linearity. */
 ORACLE_API void oracle_conv2d(const float *x, const float *w, const float *bias, const float *add, float *y, int64_t N,
                    int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t OH, int64_t OW,
                    int64_t PHL, int64_t PWL, int64_t SH, int64_t SW, int64_t DH, int64_t DW, int relu) {
@@ -567,7 +571,9 @@ ORACLE_API void oracle_conv2d(const float *x, const float *w, const float *bias,
 
 /* method 0: maximum over the taps inside the image (padding ignored, NaN taps
  * ignored: CUDNN_NOT_PROPAGATE_NAN); method 1: sum of the taps inside the image
- * divided by KH*KW (CUDNN_POOLING_AVERAGE_COUNT_INCLUDE_PADDING, Ops.cu:345-351). */
+ * divided by KH*KW (CUDNN_POOLING_AVERAGE_COUNT_INCLUDE_PADDING, Ops.cu:345-351).
+ * Pinned by tests/test_oracle_conv_pool.py: torch CPU max_pool2d / avg_pool2d
+ * on explicitly padded inputs, hand-computed cases. */
 ORACLE_API void oracle_pool2d(const float *x, float *y, int64_t planes, int64_t H, int64_t W, int64_t OH, int64_t OW,
                    int64_t KH, int64_t KW, int64_t PHL, int64_t PWL, int64_t SH, int64_t SW, int method) {
 #pragma omp parallel for schedule(static)
