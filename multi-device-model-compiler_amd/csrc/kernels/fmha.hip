@@ -42,17 +42,19 @@
 // flops, i.e. 16 issue cycles per wavefront, and a wavefront issues in order:
 // VALU work is free only while it sits between MFMAs whose results it does not
 // need.  So the per-score work is trimmed to one fma, one exp2, half a convert
-// and half a dot2, and the row maximum is taken out of the hot path entirely:
+// and one add, and the row maximum is taken out of the hot path entirely:
 //   * m is a stale reference, not the running maximum.  P is produced
 //     optimistically against it; fp16 holds p up to 2^16, and an overflow (or
-//     the first tile, where m = -inf) shows up as a non-finite row sum.  Only
+//     the first tile, where m = -inf) shows up as a row sum beyond 2^15.  Only
 //     then does the wavefront take the slow path: true row maximum, rescale of
 //     O and l, P recomputed.  O / l does not depend on which m was used.
 //     Without the maximum in front of it the softmax of a tile is a single pass
-//     of fma / exp2 / convert / dot2 over the scores;
-//   * the row sum is taken with v_dot2_f32_{f16,bf16} over the already converted
-//     P pairs (two scores per instruction; the normaliser then matches the P
-//     the matrix cores consume);
+//     of fma / exp2 / add / convert over the scores;
+//   * the row sum is a plain fp32 add per score.  v_dot2_f32_f16 over the
+//     converted P pairs would halve the instruction count, but it runs on the
+//     matrix pipeline: measured between MFMAs it costs 6 cycles that do not
+//     overlap, where add, fma, max3 and the f16 converts overlap completely
+//     and v_exp_f32 costs about 2;
 //   * accumulators stay in VGPRs (no AGPR copies);
 //   * three wavefronts share a SIMD (142 VGPRs) and are left to drift apart, so
 //     that one is in an MFMA phase while another does its softmax; s_setprio
@@ -97,7 +99,10 @@ template <int D> struct Geo {
   __host__ __device__ static constexpr int kSwz(int row) { return D == 64 ? ((row >> 1) & 7) : (row & 15); }
   __host__ __device__ static constexpr int vSwz(int row) { return D == 64 ? (((row >> 1) & 1) << 2) : ((row & 3) << 2); }
 };
-constexpr float kSumLimit = 1e30f; // a row sum above this (or NaN) means P overflowed against the stale m
+// A lane's share of a tile's row sum above this (or NaN) sends the wavefront to
+// the repair path: any p beyond the fp16 range (65504) pushes the fp32 sum past
+// it, and a legitimate sum that large only costs one needless repair.
+constexpr float kSumLimit = 32768.0f;
 
 template <typename T> struct Mma;
 template <> struct Mma<_Float16> {
@@ -111,13 +116,6 @@ template <> struct Mma<_Float16> {
   __device__ static __forceinline__ v4 readTr(const lds_u8 *p) {
     return __builtin_bit_cast(v4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 __attribute__((address_space(3))) *)p));
   }
-  // acc + sum of the two packed values of word w of a v8
-  __device__ static __forceinline__ float pairSum(v8 p, int w, float acc) {
-    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    const h2 pair = {p[2 * w], p[2 * w + 1]};
-    const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
-    return __builtin_amdgcn_fdot2(pair, ones, acc, false);
-  }
 };
 template <> struct Mma<bf16_t> {
   using v8 = bf16x8;
@@ -129,12 +127,6 @@ template <> struct Mma<bf16_t> {
   __device__ static __forceinline__ float widen(__bf16 h) { return (float)h; }
   __device__ static __forceinline__ v4 readTr(const lds_u8 *p) {
     return __builtin_bit_cast(v4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 __attribute__((address_space(3))) *)p));
-  }
-  __device__ static __forceinline__ float pairSum(v8 p, int w, float acc) {
-    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
-    const b2 pair = {p[2 * w], p[2 * w + 1]};
-    const b2 ones = {(__bf16)1.0f, (__bf16)1.0f};
-    return __builtin_amdgcn_fdot2_f32_bf16(pair, ones, acc, false);
   }
 };
 
@@ -370,21 +362,22 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_kernel(const uint16_t *__rest
       // ---- P against the stale reference maximum ---------------------------
       auto makeP = [&](float mref) {
         const float mc = mref * scale_log2e;
-        float lsum = 0.0f;
+        float lsum = 0.0f, lsumOdd = 0.0f;
 #pragma unroll
         for (int kb = 0; kb < G::KB; kb++)
 #pragma unroll
           for (int m = 0; m < 2; m++) {
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-              pf[qi][kb][m][j] = M::narrow(__builtin_amdgcn_exp2f(accS[qi][kb][8 * m + j] * scale_log2e - mc));
-#pragma unroll
-            for (int w = 0; w < 4; w++) lsum = M::pairSum(pf[qi][kb][m], w, lsum);
+            for (int j = 0; j < 8; j++) {
+              const float e = __builtin_amdgcn_exp2f(accS[qi][kb][8 * m + j] * scale_log2e - mc);
+              (j & 1 ? lsumOdd : lsum) += e;
+              pf[qi][kb][m][j] = M::narrow(e);
+            }
           }
-        return lsum;
+        return lsum + lsumOdd;
       };
       float lsum = makeP(m_run[qi]);
-      // Overflow of P (or m = -inf on the first tile) makes the sum non-finite.
+      // Overflow of P (or m = -inf on the first tile) pushes the sum past the limit.
       if (__builtin_amdgcn_ballot_w64(!(lsum <= kSumLimit)) != 0) {
         float mx = accS[qi][0][0];
 #pragma unroll

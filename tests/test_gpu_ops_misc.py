@@ -76,8 +76,10 @@ def test_matmul_f32(pkg, gpu, oracle, rng):
 
 
 def layer_tol(ref):
-    """fp16 output of an O(1..4)-magnitude tensor after ~6 fp16-rounded stages."""
-    return 2e-3 + 4e-3 * np.abs(ref)
+    """fp16 output of an O(1..4)-magnitude tensor after ~6 fp16-rounded stages.  The floor is
+    one fp16 spacing of the residual stream (2^-8 for |x| in [4, 8)): an intermediate rounded
+    the other way survives into an output that the last addition brings close to zero."""
+    return 5e-3 + 4e-3 * np.abs(ref)
 
 
 def test_bert_encoder_layer_config4(pkg, gpu, oracle):

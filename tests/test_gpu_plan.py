@@ -59,7 +59,7 @@ def test_layernorm_and_attention_plans_at_config_size(pkg, gpu, tmp_path, oracle
 
 
 def layer_tol(ref):
-    return 2e-3 + 4e-3 * np.abs(ref)
+    return 5e-3 + 4e-3 * np.abs(ref)  # see tests/test_gpu_ops_misc.py
 
 
 def test_bert_layer_composed_from_primitive_ops(pkg, gpu, tmp_path, oracle):
