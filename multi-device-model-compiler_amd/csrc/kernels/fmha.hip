@@ -43,13 +43,17 @@
 // VALU work is free only while it sits between MFMAs whose results it does not
 // need.  So the per-score work is trimmed to one fma, one exp2, half a convert
 // and one add, and the row maximum is taken out of the hot path entirely:
-//   * m is a stale reference, not the running maximum.  P is produced
-//     optimistically against it; fp16 holds p up to 2^16, and an overflow (or
-//     the first tile, where m = -inf) shows up as a row sum beyond 2^15.  Only
+//   * m is a stale reference, not the running maximum, and starts at 0.  P is
+//     produced optimistically against it; fp16 holds p up to 2^16 with the
+//     same relative precision everywhere above 2^-14, so any reference within
+//     about +-12 (base-2 units) of the true row maximum is as good as the
+//     maximum itself.  A reference that is too low shows up as a tile row sum
+//     beyond 2^15, an initial one that is too high as a first sum below 2^-6.  Only
 //     then does the wavefront take the slow path: true row maximum, rescale of
-//     O and l, P recomputed.  O / l does not depend on which m was used.
-//     Without the maximum in front of it the softmax of a tile is a single pass
-//     of fma / exp2 / add / convert over the scores;
+//     O and l (or a restart, if nothing has been accumulated yet), P
+//     recomputed.  O / l does not depend on which m was used.  Ordinary
+//     logits (|s * scale| up to ~8) never leave the fast path, whose softmax
+//     is a single pass of fma / exp2 / add / convert over the scores;
 //   * the row sum is a plain fp32 add per score.  v_dot2_f32_f16 over the
 //     converted P pairs would halve the instruction count, but it runs on the
 //     matrix pipeline: measured between MFMAs it costs 6 cycles that do not
@@ -99,10 +103,18 @@ template <int D> struct Geo {
   __host__ __device__ static constexpr int kSwz(int row) { return D == 64 ? ((row >> 1) & 7) : (row & 15); }
   __host__ __device__ static constexpr int vSwz(int row) { return D == 64 ? (((row >> 1) & 1) << 2) : ((row & 3) << 2); }
 };
-// A lane's share of a tile's row sum above this (or NaN) sends the wavefront to
-// the repair path: any p beyond the fp16 range (65504) pushes the fp32 sum past
-// it, and a legitimate sum that large only costs one needless repair.
+// A lane's share of a tile's row sum above kSumLimit (or NaN) sends the
+// wavefront to the repair path: any p beyond the fp16 range (65504) pushes the
+// fp32 sum past it, and a legitimate sum that large only costs one needless
+// repair.  A sum below kSumFloor on the first tile means the initial reference
+// sits so far above the scores that P is leaving fp16's normal range (the
+// largest p of a row is at least sum / keys): the reference is then lowered to
+// the tile's maximum.  Every query sees a key in the first tile (key 0 is
+// valid under both masks), so from then on its running sum stays above the
+// floor - a raised reference comes with a tile whose largest p is 1 - and the
+// test is not needed again.
 constexpr float kSumLimit = 32768.0f;
+constexpr float kSumFloor = 0.015625f;
 
 template <typename T> struct Mma;
 template <> struct Mma<_Float16> {
@@ -277,10 +289,10 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_kernel(const uint16_t *__rest
   }
 
   f32x16 accO[NQ][G::DB];
-  float m_run[NQ], l_run[NQ]; // stale reference maximum (raw score units), running sum
+  float m_run[NQ], l_run[NQ]; // stale reference maximum (raw score units), this lane's share of the running sum
 #pragma unroll
   for (int qi = 0; qi < NQ; qi++) {
-    m_run[qi] = -INFINITY;
+    m_run[qi] = 0.0f;
     l_run[qi] = 0.0f;
 #pragma unroll
     for (int db = 0; db < G::DB; db++)
@@ -377,17 +389,22 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_kernel(const uint16_t *__rest
         return lsum + lsumOdd;
       };
       float lsum = makeP(m_run[qi]);
-      // Overflow of P (or m = -inf on the first tile) pushes the sum past the limit.
-      if (__builtin_amdgcn_ballot_w64(!(lsum <= kSumLimit)) != 0) {
+      // Reference too low (P overflows) or too high (everything so far underflows).
+      if (__builtin_amdgcn_ballot_w64(!(lsum <= kSumLimit) || (kt == 0 && !(lsum >= kSumFloor))) != 0) {
         float mx = accS[qi][0][0];
 #pragma unroll
         for (int kb = 0; kb < G::KB; kb++)
 #pragma unroll
           for (int i = 0; i < 16; i++) mx = fmaxf(mx, accS[qi][kb][i]);
         mx = halves_max(mx);
-        const float m_new = fmaxf(m_run[qi], mx);
-        // rows that never saw a key yet have l = 0 and O = 0: any finite factor does
-        const float alpha = m_run[qi] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f((m_run[qi] - m_new) * scale_log2e);
+        float m_new, alpha;
+        if (kt > 0) { // the row has a history: the reference only rises
+          m_new = fmaxf(m_run[qi], mx);
+          alpha = __builtin_amdgcn_exp2f((m_run[qi] - m_new) * scale_log2e);
+        } else { // first tile: start over from its maximum
+          m_new = mx == -INFINITY ? m_run[qi] : mx;
+          alpha = 0.0f;
+        }
         m_run[qi] = m_new;
         l_run[qi] *= alpha;
 #pragma unroll

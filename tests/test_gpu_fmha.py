@@ -104,6 +104,34 @@ def test_fmha_large_logits_and_other_scales(pkg, gpu, oracle, rng):
     assert excess(run(pkg, gpu, qkv, scale=1.0), oracle.fmha(qkv, scale=1.0), TOL_F16) <= 1.0
 
 
+@pytest.mark.parametrize("D", [64, 128])
+def test_fmha_logits_far_from_zero(pkg, gpu, oracle, rng, D):
+    """The kernel's first softmax reference is 0.  Logits that all sit far below
+    it (every p underflows on the first pass) or far above it (every p
+    overflows) must be caught on the first tile; a common offset of all of a
+    row's logits does not change the softmax."""
+    B, S, H = 1, 200, 2
+    qkv = make_qkv(rng, B, S, H, std=0.5, D=D)
+    u = np.zeros(D, np.float16)
+    u[:8] = 4.0
+    for sign in (-1.0, 1.0):  # q.k moves by -+128: logits near -+16 (D = 64) or -+11 (D = 128) plus noise
+        shifted = qkv.copy()
+        shifted[:, :, 0, 0, :] += np.float16(sign) * u   # queries of head 0
+        shifted[:, :, 1, 0, :] += u                      # keys of head 0
+        ref = oracle.fmha(shifted)
+        got = run(pkg, gpu, shifted)
+        assert np.isfinite(got).all() and excess(got, ref, TOL_F16) <= 1.0, sign
+    # first tile far below the reference, later keys far above the first tile
+    ramp = qkv.copy()
+    ramp[:, :, 0, :, :] = 0
+    ramp[:, :, 0, :, 0] = 8.0
+    ramp[:, :, 1, :, 0] = np.linspace(-60.0, 60.0, S, dtype=np.float16)[None, :, None]
+    for causal in (False, True):
+        ref = oracle.fmha(ramp, causal=causal)
+        got = run(pkg, gpu, ramp, causal=causal)
+        assert np.isfinite(got).all() and excess(got, ref, TOL_F16) <= 1.0, causal
+
+
 @pytest.mark.parametrize("B,S,H,lens,causal", [
     (2, 128, 8, None, False), (1, 1, 1, None, False), (2, 31, 2, None, False), (1, 32, 1, None, True),
     (2, 33, 2, [33, 7], False), (1, 257, 3, None, True), (2, 512, 2, [512, 300], False), (3, 100, 2, [0, 1, 100], True),
