@@ -40,10 +40,21 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 MALL_BYTES = 256 << 20
-# HBM bytes per launch of the headline kernel, from two rocprofv3 --pmc passes
+# HBM bytes per launch, from two rocprofv3 --pmc passes over this script
 # (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0, the factors a 64 MiB device copy
-# gives for the same counters); see profiles/layernorm_f32_hbm_traffic.md.
+# gives for the same counters); see profiles/layernorm_f32_hbm_traffic.md for the
+# headline kernel and profiles/bench_all_configs_hbm_traffic.md for the others.
 LN_F32_TRAFFIC_BYTES = 25_250_000
+TRAFFIC_BYTES = {
+    "layernorm_f16": 12_655_000,
+    "add_f32": 14_762_000,
+    "layernorm_f32_large": 1_610_400_000,
+    "add_f32_large": 3_220_200_000,
+    "fmha_b32_s128": 25_310_000,
+    "fmha_b8_s512_masked": 31_870_000,
+    "fmha_b32_s512": 100_780_000,
+    "fmha_d128_b32_s512": 134_300_000,
+}
 
 
 def parse_args():
@@ -104,6 +115,38 @@ class Timer:
             return e0.elapsed_time(e1)
 
 
+def device_info(torch) -> dict:
+    """What the device reports about itself, with the peaks those figures imply:
+    dense fp16 MFMA = CUs x 4 SIMDs x 1024 flop/clock x shader clock, HBM =
+    2 transfers/clock x memory clock x bus width.  The roofline objects use the
+    published 2.5 PFLOP/s and 8 TB/s; these are printed beside them."""
+    pr = torch.cuda.get_device_properties(0)
+    cus = getattr(pr, "multi_processor_count", None)
+    clk_khz = getattr(pr, "clock_rate", None)
+    mclk_khz = getattr(pr, "memory_clock_rate", None)
+    bus = getattr(pr, "memory_bus_width", None)
+    info = {"arch": getattr(pr, "gcnArchName", None), "compute_units": cus, "shader_clock_mhz": clk_khz and clk_khz / 1e3,
+            "memory_clock_mhz": mclk_khz and mclk_khz / 1e3, "memory_bus_bits": bus,
+            "hbm_bytes": getattr(pr, "total_memory", None)}
+    try:  # torch does not report clocks on this platform; the runtime's own listing does
+        import re
+        import subprocess
+        txt = subprocess.run(["/opt/rocm/bin/rocminfo"], capture_output=True, text=True, timeout=30).stdout
+        for agent in txt.split("*******")[1:]:
+            if "gfx950" in agent and "Max Clock Freq. (MHz)" in agent:
+                mhz = float(re.search(r"Max Clock Freq\. \(MHz\):\s*(\d+)", agent).group(1))
+                info["shader_clock_mhz"] = info["shader_clock_mhz"] or mhz
+                clk_khz = clk_khz or mhz * 1e3
+                break
+    except Exception:
+        pass
+    if cus and clk_khz:
+        info["mfma_f16_peak_tflops_at_reported_clock"] = round(cus * 4 * 1024 * clk_khz * 1e3 / 1e12, 1)
+    if mclk_khz and bus:
+        info["hbm_peak_gbs_at_reported_clock"] = round(2 * mclk_khz * 1e3 * bus / 8 / 1e9, 1)
+    return info
+
+
 def rotating_sets(bytes_per_set: int) -> int:
     """Number of buffer sets whose total footprint exceeds the Infinity Cache."""
     return max(2, (MALL_BYTES + bytes_per_set - 1) // bytes_per_set + 2)
@@ -115,7 +158,7 @@ def hbm_entry(name, workload, dtype, bytes_per_launch, ms, steps, warm_ms=None):
     e = {"name": name, "workload": workload, "dtype": dtype, "metric": "GB/s", "value": round(gbs, 1),
          "us_per_launch": round(us, 3),
          "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES.get(name)},
          "algorithmic_bytes": bytes_per_launch}
     if warm_ms is not None:
         wus = warm_ms * 1e3 / steps
@@ -318,7 +361,8 @@ def main():
         entry = {"name": name, "workload": workload, "dtype": "f16", "metric": "TFLOP/s", "value": round(tf, 1),
                  "us_per_launch": round(us, 3),
                  "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_F16_PEAK_TFLOPS,
-                              "unit": "TFLOP/s", "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+                              "unit": "TFLOP/s", "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                              "traffic": TRAFFIC_BYTES.get(name)},
                  "algorithmic_flop": flop_valid, "algorithmic_bytes": nbytes,
                  "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
         if masked:
@@ -397,6 +441,7 @@ def main():
         "roofline": headline["roofline"], "cache_resident": headline.get("cache_resident"),
         "cpu_baseline": cpu, "kernels": kernels,
         "device": torch.cuda.get_device_name(0),
+        "device_info": device_info(torch),
     }
     print(json.dumps(result))
 
