@@ -18,9 +18,11 @@
 
 #include <hipblaslt/hipblaslt.h>
 
+#include <algorithm>
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <vector>
 
 namespace mgpu {
 
@@ -65,7 +67,8 @@ void destroyPlan(Plan &p) {
   p = Plan{};
 }
 
-constexpr int kCandidates = 16;
+constexpr int kCandidates = 64; // heuristic answers asked for and screened
+constexpr int kFinalists = 4;   // re-timed at length after the screening pass
 
 // Times the candidates on scratch operands of the plan's shape (its own stream,
 // its own buffers: the caller's data and stream are not touched) and returns
@@ -90,11 +93,10 @@ int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *resu
     if (hasBias)
       (void)hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
     const float alpha = 1.0f, beta = hasResidual ? 1.0f : 0.0f;
-    float bestMs = -1.0f;
-    for (int c = 0; c < count; c++) {
-      if (results[c].state != HIPBLAS_STATUS_SUCCESS || results[c].workspaceSize > workspaceSize) continue;
+    // reps launches of candidate c between two events, after one untimed launch; < 0 on failure
+    auto timeCandidate = [&](int c, int reps) -> float {
       bool ok = true;
-      for (int rep = 0; rep < 6 && ok; rep++) { // one untimed, five timed
+      for (int rep = 0; rep <= reps && ok; rep++) {
         if (rep == 1) (void)hipEventRecord(e0, s);
         ok = hipblasLtMatmul(ltHandle, p.op, &alpha, w, p.a, in, p.b, &beta, out, p.d, out, p.d, &results[c].algo,
                              workspace, workspaceSize, s) == HIPBLAS_STATUS_SUCCESS;
@@ -102,10 +104,24 @@ int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *resu
       float ms = 0.0f;
       if (!ok || hipEventRecord(e1, s) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
           hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
-        continue;
-      if (bestMs < 0.0f || ms < bestMs) {
+        return -1.0f;
+      return ms / reps;
+    };
+    // Screening: three launches each; the kFinalists fastest go on.
+    std::vector<std::pair<float, int>> screened;
+    for (int c = 0; c < count; c++) {
+      if (results[c].state != HIPBLAS_STATUS_SUCCESS || results[c].workspaceSize > workspaceSize) continue;
+      const float ms = timeCandidate(c, 3);
+      if (ms >= 0.0f) screened.emplace_back(ms, c);
+    }
+    std::sort(screened.begin(), screened.end());
+    // Final: twenty launches each.
+    float bestMs = -1.0f;
+    for (size_t i = 0; i < screened.size() && i < (size_t)kFinalists; i++) {
+      const float ms = timeCandidate(screened[i].second, 20);
+      if (ms >= 0.0f && (bestMs < 0.0f || ms < bestMs)) {
         bestMs = ms;
-        best = c;
+        best = screened[i].second;
       }
     }
     (void)hipStreamSynchronize(s);
