@@ -144,6 +144,20 @@ def test_gpu_runner_add_model_matches_cpu_runner(pkg, gpu, tmp_path, oracle):
     assert np.array_equal(outs["gpu"].view(np.uint32), oracle.add_f32(a, b).reshape(-1).view(np.uint32))
 
 
+def test_gpu_runner_runs_what_lib_generate_emitted(pkg, gpu, tmp_path, oracle):
+    """The add model and its kernel module after multi-device-lib-generate took
+    them from LLVM IR (host: opt -> llc -> .so, kernel: AMDGPU IR -> ops.hsaco)."""
+    gen = os.path.join(pkg.LIB_DIR, "models", "generated")
+    a = gen_data.gen_data("3_640_640", seed=31, dist="uniform")
+    b = gen_data.gen_data("3_640_640", seed=32, dist="uniform")
+    fa, fb = gen_data.save_data(a, str(tmp_path / "a")), gen_data.save_data(b, str(tmp_path / "b"))
+    out = str(tmp_path / "c.dat")
+    r = subprocess.run([_runner(pkg, "multi-device-gpu-runner"), os.path.join(gen, "add_gpu.so"), "--ops",
+                        os.path.join(gen, "ops.hsaco"), "--data", f"{fa},{fb}", "--out-data", out],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.fromfile(out, np.float32).view(np.uint32), oracle.add_f32(a, b).reshape(-1).view(np.uint32))
+
 def test_gpu_runner_layernorm_and_fmha_models(pkg, gpu, tmp_path, oracle):
     x = gen_data.gen_data("32_128_768", seed=1, dist="normal")
     g = gen_data.gen_data("768", seed=2, dist="normal", mean=1.0, std=0.02)

@@ -150,3 +150,61 @@ def test_gpu_runner_links_and_prints_help(paths):
     assert r.returncode == 0
     for flag in ("--func", "--out-data", "--rerun", "--ops", "--input", "--output", "--data", "--dtype"):
         assert flag in r.stdout
+
+
+def test_lib_generate_cpu_model_from_llvm_ir(paths, pkg, tmp_path, oracle):
+    """multi-device-lib-generate (the reference's tool of that name,
+    tools/multi-device-lib-generate/multi-device-lib-generate.cpp:41-67): model
+    LLVM IR -> opt -> llc -> shared library, temporaries removed unless asked
+    for, and the library runs under the CPU runner."""
+    import shutil
+    tool = os.path.join(pkg.BIN_DIR, "multi-device-lib-generate")
+    gen = os.path.join(paths["models"], "generated")
+    # the build already took the add model through the tool; that library must run
+    a = gen_data.gen_data("2_33_65", seed=5, dist="uniform")
+    b = gen_data.gen_data("2_33_65", seed=6, dist="uniform")
+    fa, fb = gen_data.save_data(a, str(tmp_path / "a")), gen_data.save_data(b, str(tmp_path / "b"))
+    out = str(tmp_path / "c.dat")
+    r = run([paths["cpu_runner"], os.path.join(gen, "add_cpu.so"), "--input", "2_33_65,2_33_65", "--output", "2_33_65",
+             "--data", f"{fa},{fb}", "--out-data", out])
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.fromfile(out, np.float32).view(np.uint32), oracle.add_f32(a, b).reshape(-1).view(np.uint32))
+    # a fresh run of the tool on the same IR, in a scratch directory
+    ll = str(tmp_path / "model.ll")
+    shutil.copy(os.path.join(gen, "add_cpu.ll"), ll)
+    r = run([tool, ll, "--saveObject"])
+    assert r.returncode == 0, r.stderr
+    assert os.path.exists(tmp_path / "model.so") and os.path.exists(tmp_path / "model.o")
+    assert not os.path.exists(tmp_path / "model_opt.ll")
+    r = run([tool, ll, "-o", str(tmp_path / "named"), "--saveOptIR", "-O3"])
+    assert r.returncode == 0, r.stderr
+    assert os.path.exists(tmp_path / "named.so") and os.path.exists(tmp_path / "model_opt.ll")
+    r = run([paths["cpu_runner"], str(tmp_path / "named.so"), "--input", "2_33_65,2_33_65", "--output", "2_33_65",
+             "--data", f"{fa},{fb}", "--out-data", out])
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.fromfile(out, np.float32).view(np.uint32), oracle.add_f32(a, b).reshape(-1).view(np.uint32))
+    # an invalid -o is ignored with a note, as the reference does (:157-166)
+    r = run([tool, ll, "-o", str(tmp_path) + "/.."])
+    assert r.returncode == 0 and "Invalid -o option value" in r.stderr
+
+
+def test_lib_generate_gpu_artifacts_and_errors(pkg, paths, tmp_path):
+    """--device gpu also turns the kernel source (AMDGPU LLVM IR or HIP) into
+    ops.hsaco beside it; the build's own run of it left a code object holding the
+    generated-style kernel.  Failures name the step and return non-zero."""
+    tool = os.path.join(pkg.BIN_DIR, "multi-device-lib-generate")
+    gen = os.path.join(paths["models"], "generated")
+    blob = open(os.path.join(gen, "ops.hsaco"), "rb").read()
+    assert blob[:4] == b"\x7fELF" and b"main_graph_kernel" in blob
+    assert os.path.exists(os.path.join(gen, "add_gpu.so"))
+    r = run([tool, str(tmp_path / "missing.ll")])
+    assert r.returncode != 0 and "Failed to open input" in r.stderr
+    bad = tmp_path / "bad.ll"
+    bad.write_text("this is not LLVM IR\n")
+    r = run([tool, str(bad)])
+    assert r.returncode != 0 and "Opt LLVM IR wrong." in r.stderr and "Command execution failed." in r.stderr
+    r = run([tool, os.path.join(gen, "add_cpu.ll"), "-o", str(tmp_path / "x"), "--device", "tpu"])
+    assert r.returncode != 0 and "--device is cpu or gpu" in r.stderr
+    r = run([tool, os.path.join(gen, "add_gpu.ll"), "-o", str(tmp_path / "y"), "--device", "gpu",
+             "--ops", str(tmp_path / "nope.hip")])
+    assert r.returncode != 0 and "kernel source not found" in r.stderr
