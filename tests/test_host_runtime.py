@@ -208,3 +208,26 @@ def test_lib_generate_gpu_artifacts_and_errors(pkg, paths, tmp_path):
     r = run([tool, os.path.join(gen, "add_gpu.ll"), "-o", str(tmp_path / "y"), "--device", "gpu",
              "--ops", str(tmp_path / "nope.hip")])
     assert r.returncode != 0 and "kernel source not found" in r.stderr
+
+
+REF_ADD_LL = "/root/reference/examples/add.ll"
+
+
+@pytest.mark.skipif(not os.path.exists(REF_ADD_LL), reason="the reference tree is not present on this machine")
+def test_reference_add_ll_through_lib_generate_and_cpu_runner(pkg, paths, tmp_path, oracle):
+    """The reference's one pre-lowered model (examples/add.ll:8-104, entry
+    _mlir_ciface_main_graph with outputs first) goes through this build's
+    multi-device-lib-generate and runs under this build's CPU runner with the
+    reference's own default shapes; the result is bit-exact."""
+    import shutil
+    ll = str(tmp_path / "add.ll")
+    shutil.copy(REF_ADD_LL, ll)
+    r = run([os.path.join(pkg.BIN_DIR, "multi-device-lib-generate"), ll, "-o", str(tmp_path / "add")])
+    assert r.returncode == 0, r.stderr
+    a = gen_data.gen_data("3_640_640", seed=41, dist="uniform")
+    b = gen_data.gen_data("3_640_640", seed=42, dist="uniform")
+    fa, fb = gen_data.save_data(a, str(tmp_path / "a")), gen_data.save_data(b, str(tmp_path / "b"))
+    out = str(tmp_path / "c.dat")
+    r = run([paths["cpu_runner"], str(tmp_path / "add.so"), "--data", f"{fa},{fb}", "--out-data", out, "--rerun", "2"])
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.fromfile(out, np.float32).view(np.uint32), oracle.add_f32(a, b).reshape(-1).view(np.uint32))
