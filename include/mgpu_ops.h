@@ -101,6 +101,9 @@ void mgpuFusedMHABF16(const void *qkv, const int32_t *seqlens, void *out, int32_
 /* ---- casts (Utils.h:6-8; lib/Kernels/GPU/Utils.cu:85-103) ------------- */
 void mgpuCastF32ToF16(void *dst, const float *src, size_t size, mgpuStream_t stream);
 void mgpuCastF16ToF32(float *dst, const void *src, size_t size, mgpuStream_t stream);
+/* bfloat16 counterparts (16-bit patterns; round to nearest even, NaN kept quiet). */
+void mgpuCastF32ToBF16(void *dst, const float *src, size_t size, mgpuStream_t stream);
+void mgpuCastBF16ToF32(float *dst, const void *src, size_t size, mgpuStream_t stream);
 
 /* ---- QKV bias + transpose (Ops.h:70-74; Transpose.cu:70-84) ----------- */
 /* QKV [token,3,H,D] += bias[3,H,D] in place; q/k/v_buf receive [B,H,S,D]. */
@@ -108,6 +111,10 @@ void mgpuAddFusedQKVBiasTransposeF16(void *q_buf, void *k_buf, void *v_buf, void
                                      const void *qkv_bias, int32_t batch_size, int32_t seq_len,
                                      int32_t token_num, int32_t head_num, int32_t size_per_head,
                                      mgpuStream_t stream);
+void mgpuAddFusedQKVBiasTransposeBF16(void *q_buf, void *k_buf, void *v_buf, void *QKV,
+                                      const void *qkv_bias, int32_t batch_size, int32_t seq_len,
+                                      int32_t token_num, int32_t head_num, int32_t size_per_head,
+                                      mgpuStream_t stream);
 
 /* ---- GEMM ------------------------------------------------------------- */
 /* output[M,N] = input[M,K] . weight[K,N] + bias[N], fp32, row major
@@ -139,6 +146,9 @@ void mgpuMatmulExF16(void *input, void *weight, void *bias, void *output, void *
 void mgpuMatmulExF32(float *input, float *weight, float *bias, float *output, float *residual,
                      int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
                      int32_t hasResidual, mgpuStream_t stream);
+void mgpuMatmulExBF16(void *input, void *weight, void *bias, void *output, void *residual,
+                      int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
+                      int32_t hasResidual, mgpuStream_t stream);
 
 /* ---- transformer layers ----------------------------------------------- */
 /* Pre-LN layer, fp32 in/out, fp16 compute; same signature as the reference

@@ -58,11 +58,15 @@ OPS_SIGNATURES = {
     "mgpuFusedMHABF16": (None, [_c_void_p] * 3 + [_c_int32] * 4 + [_c_float, _c_int32, _c_void_p]),
     "mgpuCastF32ToF16": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
     "mgpuCastF16ToF32": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
+    "mgpuCastF32ToBF16": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
+    "mgpuCastBF16ToF32": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
     "mgpuAddFusedQKVBiasTransposeF16": (None, [_c_void_p] * 5 + [_c_int32] * 5 + [_c_void_p]),
+    "mgpuAddFusedQKVBiasTransposeBF16": (None, [_c_void_p] * 5 + [_c_int32] * 5 + [_c_void_p]),
     "mgpuMatmul": (None, [_c_void_p] * 4 + [_c_int64] * 3 + [_c_void_p]),
     "mgpuConv2d": (None, [_c_void_p] * 5 + [_c_int64] * 17 + [ctypes.c_bool] * 2 + [_c_void_p]),
     "mgpuPool2d": (None, [_c_void_p] * 2 + [_c_int64] * 15 + [_c_void_p]),
     "mgpuMatmulExF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
+    "mgpuMatmulExBF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuMatmulExF32": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuLLMDecodingContextLayer": (None, [_c_void_p] * 9 + [_c_int64] * 5 + [ctypes.c_bool] * 3 + [_c_void_p]),
     "mgpuBertEncoderLayerF16": (None, [_c_void_p] * 15 + [_c_int64] * 5 + [_c_float, _c_void_p]),
@@ -244,16 +248,34 @@ def cast_f16_to_f32(x, stream=None):
     return out
 
 
+def cast_f32_to_bf16(x, stream=None):
+    import torch
+    out = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    lib = ops()
+    lib.mgpuCastF32ToBF16(_ptr(out), _ptr(x), x.numel(), _stream_handle(stream))
+    _check(lib)
+    return out
+
+
+def cast_bf16_to_f32(x, stream=None):
+    import torch
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    lib = ops()
+    lib.mgpuCastBF16ToF32(_ptr(out), _ptr(x), x.numel(), _stream_handle(stream))
+    _check(lib)
+    return out
+
+
 def qkv_bias_transpose(qkv, bias, stream=None):
-    """qkv [B,S,3,H,D] fp16 (updated in place with the bias) -> q, k, v [B,H,S,D]."""
+    """qkv [B,S,3,H,D] fp16 or bf16 (updated in place with the bias) -> q, k, v [B,H,S,D]."""
     import torch
     B, S, _, H, D = qkv.shape
     q = torch.empty((B, H, S, D), dtype=qkv.dtype, device=qkv.device)
     k = torch.empty_like(q)
     v = torch.empty_like(q)
     lib = ops()
-    lib.mgpuAddFusedQKVBiasTransposeF16(_ptr(q), _ptr(k), _ptr(v), _ptr(qkv), _ptr(bias), B, S,
-                                        B * S, H, D, _stream_handle(stream))
+    fn = lib.mgpuAddFusedQKVBiasTransposeBF16 if qkv.dtype == torch.bfloat16 else lib.mgpuAddFusedQKVBiasTransposeF16
+    fn(_ptr(q), _ptr(k), _ptr(v), _ptr(qkv), _ptr(bias), B, S, B * S, H, D, _stream_handle(stream))
     _check(lib)
     return q, k, v
 
@@ -268,7 +290,8 @@ def matmul_ex(x, w, bias=None, residual=None, act: int = ACT_NONE, stream=None):
     assert K == K2
     out = torch.empty((M, N), dtype=x.dtype, device=x.device)
     lib = ops()
-    fn = lib.mgpuMatmulExF16 if x.dtype == torch.float16 else lib.mgpuMatmulExF32
+    fn = {torch.float16: lib.mgpuMatmulExF16, torch.bfloat16: lib.mgpuMatmulExBF16,
+          torch.float32: lib.mgpuMatmulExF32}[x.dtype]
     fn(_ptr(x), _ptr(w), _ptr(bias), _ptr(out), _ptr(residual), M, N, K,
        1 if bias is not None else 0, act, 1 if residual is not None else 0, _stream_handle(stream))
     _check(lib)

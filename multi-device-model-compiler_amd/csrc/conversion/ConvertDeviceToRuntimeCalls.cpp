@@ -203,8 +203,10 @@ bool emitOp(Lowering &L, const DeviceOp &op, std::string &error) {
   }
   if (n == "device.cast") {
     if (!gpu) return noCpu();
-    L.call(inT(0).elem == ElemType::F32 ? "mgpuCastF32ToF16" : "mgpuCastF16ToF32",
-           withStream({out(0), in(0), i64(inT(0).numel())}));
+    const ElemType from = inT(0).elem, to = plan.values[op.results[0]].type.elem;
+    const char *callee = from == ElemType::F32 ? (to == ElemType::BF16 ? "mgpuCastF32ToBF16" : "mgpuCastF32ToF16")
+                                               : (from == ElemType::BF16 ? "mgpuCastBF16ToF32" : "mgpuCastF16ToF32");
+    L.call(callee, withStream({out(0), in(0), i64(inT(0).numel())}));
     return true;
   }
   if (n == "device.fused-mha") {

@@ -449,7 +449,7 @@ bool verifyOp(const DevicePlan &plan, const DeviceOp &op, std::string &error) {
   }
   if (n == "device.matmul-ex") {
     if (!v.counts(4, 1) || !v.required({0, 1}) || !v.attrKinds({{"act", AttrValue::String}})) return false;
-    if (v.in(0).elem != ElemType::F32 && v.in(0).elem != ElemType::F16) return v.fail("built for f32 and f16");
+    if (!isFloat(v.in(0).elem)) return v.fail("built for f32, f16 and bf16");
     if (!verifyMatmulShapes(v, v.present(2))) return false;
     if (v.present(3) && v.in(3) != v.out(0)) return v.fail("residual has the type of the result");
     auto act = op.attrs.find("act");
@@ -524,8 +524,9 @@ bool verifyOp(const DevicePlan &plan, const DeviceOp &op, std::string &error) {
     if (!v.counts(1, 1) || !v.required({0}) || !v.attrKinds({})) return false;
     if (v.in(0).shape != v.out(0).shape) return v.fail("result has the shape of the operand");
     const ElemType a = v.in(0).elem, b = v.out(0).elem;
-    if (!((a == ElemType::F32 && b == ElemType::F16) || (a == ElemType::F16 && b == ElemType::F32)))
-      return v.fail("casts f32 -> f16 or f16 -> f32");
+    const bool narrow = a == ElemType::F32 && (b == ElemType::F16 || b == ElemType::BF16);
+    const bool widen = b == ElemType::F32 && (a == ElemType::F16 || a == ElemType::BF16);
+    if (!narrow && !widen) return v.fail("casts f32 -> f16 / bf16 or f16 / bf16 -> f32");
     return true;
   }
   if (n == "device.fused-mha") {

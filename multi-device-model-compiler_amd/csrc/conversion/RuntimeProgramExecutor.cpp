@@ -113,7 +113,7 @@ bool dispatch(Machine &m, const RuntimeCall &c) {
     ((void (*)(P, P, P, I, I, I, I, F, I, P))fn)(p(0), p(1), p(2), i(3), i(4), i(5), i(6), f(7), i(8), p(9));
     return true;
   }
-  if (n == "mgpuCastF32ToF16" || n == "mgpuCastF16ToF32") { ((void (*)(P, P, size_t, P))fn)(p(0), p(1), (size_t)l(2), p(3)); return true; }
+  if (n == "mgpuCastF32ToF16" || n == "mgpuCastF16ToF32" || n == "mgpuCastF32ToBF16" || n == "mgpuCastBF16ToF32") { ((void (*)(P, P, size_t, P))fn)(p(0), p(1), (size_t)l(2), p(3)); return true; }
   if (n == "mgpuConv2d" || n == "mcpuConv2d") {
     typedef void (*Gpu)(P, P, P, P, P, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, bool, bool, P);
     typedef void (*Cpu)(P, P, P, P, P, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, L, bool, bool);
@@ -135,7 +135,7 @@ bool dispatch(Machine &m, const RuntimeCall &c) {
     return true;
   }
   if (n == "mgpuMatmul") { ((void (*)(P, P, P, P, L, L, L, P))fn)(p(0), p(1), p(2), p(3), l(4), l(5), l(6), p(7)); return true; }
-  if (n == "mgpuMatmulExF16" || n == "mgpuMatmulExF32") {
+  if (n == "mgpuMatmulExF16" || n == "mgpuMatmulExF32" || n == "mgpuMatmulExBF16") {
     ((void (*)(P, P, P, P, P, L, L, L, I, I, I, P))fn)(p(0), p(1), p(2), p(3), p(4), l(5), l(6), l(7), i(8), i(9), i(10), p(11));
     return true;
   }

@@ -216,6 +216,12 @@ void mgpuCastF32ToF16(void *dst, const float *src, size_t size, mgpuStream_t str
 void mgpuCastF16ToF32(float *dst, const void *src, size_t size, mgpuStream_t stream) {
   guarded([&] { mgpu::castF16ToF32(dst, src, size, S(stream)); });
 }
+void mgpuCastF32ToBF16(void *dst, const float *src, size_t size, mgpuStream_t stream) {
+  guarded([&] { mgpu::castF32ToBF16(dst, src, size, S(stream)); });
+}
+void mgpuCastBF16ToF32(float *dst, const void *src, size_t size, mgpuStream_t stream) {
+  guarded([&] { mgpu::castBF16ToF32(dst, src, size, S(stream)); });
+}
 
 void mgpuAddFusedQKVBiasTransposeF16(void *q_buf, void *k_buf, void *v_buf, void *QKV,
                                      const void *qkv_bias, int32_t batch_size, int32_t seq_len,
@@ -224,6 +230,15 @@ void mgpuAddFusedQKVBiasTransposeF16(void *q_buf, void *k_buf, void *v_buf, void
   guarded([&] {
     mgpu::addFusedQKVBiasTransposeF16(q_buf, k_buf, v_buf, QKV, qkv_bias, batch_size, seq_len,
                                       token_num, head_num, size_per_head, S(stream));
+  });
+}
+void mgpuAddFusedQKVBiasTransposeBF16(void *q_buf, void *k_buf, void *v_buf, void *QKV,
+                                      const void *qkv_bias, int32_t batch_size, int32_t seq_len,
+                                      int32_t token_num, int32_t head_num, int32_t size_per_head,
+                                      mgpuStream_t stream) {
+  guarded([&] {
+    mgpu::addFusedQKVBiasTranspose(mgpu::DType::BF16, q_buf, k_buf, v_buf, QKV, qkv_bias, batch_size, seq_len,
+                                   token_num, head_num, size_per_head, S(stream));
   });
 }
 
@@ -255,6 +270,14 @@ void mgpuMatmulExF16(void *input, void *weight, void *bias, void *output, void *
                      int32_t hasResidual, mgpuStream_t stream) {
   guarded([&] {
     mgpu::matmulEx(mgpu::DType::F16, input, weight, bias, output, residual, M, N, K, hasBias != 0,
+                   hasRelu, hasResidual != 0, S(stream));
+  });
+}
+void mgpuMatmulExBF16(void *input, void *weight, void *bias, void *output, void *residual,
+                      int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
+                      int32_t hasResidual, mgpuStream_t stream) {
+  guarded([&] {
+    mgpu::matmulEx(mgpu::DType::BF16, input, weight, bias, output, residual, M, N, K, hasBias != 0,
                    hasRelu, hasResidual != 0, S(stream));
   });
 }

@@ -1,4 +1,4 @@
-// fp32 <-> fp16 casts, constant fills and the QKV bias + head transpose.
+// fp32 <-> fp16 / bf16 casts, constant fills, the QKV bias + head transpose and GELU.
 //
 // Casts replace cudaCastFloat2Half / cudaCastHalf2Float
 // (lib/Kernels/GPU/Utils.cu:38-103): the reference stages every value through
@@ -18,37 +18,28 @@ namespace {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
-__global__ __launch_bounds__(256) void cast_f32_to_f16_vec8_kernel(f16x8 *__restrict__ dst,
-                                                                   const f32x4 *__restrict__ src,
-                                                                   size_t n8) {
+// T is the 16-bit type (_Float16 or bf16_t); its vectors travel as 16 raw bytes.
+template <typename T>
+__global__ __launch_bounds__(256) void cast_f32_to_h_vec8_kernel(u32x4 *__restrict__ dst,
+                                                                 const f32x4 *__restrict__ src, size_t n8) {
   const size_t stride = (size_t)gridDim.x * 256;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += stride) {
     const f32x4 lo = src[2 * i];
     const f32x4 hi = src[2 * i + 1];
-    f16x8 o;
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      o[e] = (_Float16)lo[e];
-      o[4 + e] = (_Float16)hi[e];
-    }
-    __builtin_nontemporal_store(o, dst + i);
+    const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    __builtin_nontemporal_store(ElemTraits<T>::pack(v), dst + i);
   }
 }
 
-__global__ __launch_bounds__(256) void cast_f16_to_f32_vec8_kernel(f32x4 *__restrict__ dst,
-                                                                   const f16x8 *__restrict__ src,
-                                                                   size_t n8) {
+template <typename T>
+__global__ __launch_bounds__(256) void cast_h_to_f32_vec8_kernel(f32x4 *__restrict__ dst,
+                                                                 const u32x4 *__restrict__ src, size_t n8) {
   const size_t stride = (size_t)gridDim.x * 256;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += stride) {
-    const f16x8 v = src[i];
-    f32x4 lo, hi;
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      lo[e] = (float)v[e];
-      hi[e] = (float)v[4 + e];
-    }
-    __builtin_nontemporal_store(lo, dst + 2 * i);
-    __builtin_nontemporal_store(hi, dst + 2 * i + 1);
+    float v[8];
+    ElemTraits<T>::unpack(src[i], v);
+    __builtin_nontemporal_store(f32x4{v[0], v[1], v[2], v[3]}, dst + 2 * i);
+    __builtin_nontemporal_store(f32x4{v[4], v[5], v[6], v[7]}, dst + 2 * i + 1);
   }
 }
 
@@ -58,7 +49,7 @@ __global__ __launch_bounds__(256) void cast_scalar_kernel(TO *__restrict__ dst,
                                                           size_t n) {
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (size_t i = begin + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
-    dst[i] = (TO)src[i];
+    dst[i] = ElemTraits<TO>::fromFloat(ElemTraits<TI>::toFloat(src[i]));
 }
 
 template <typename T>
@@ -79,14 +70,15 @@ unsigned gridFor(size_t items, int perBlock) {
 // QKV [token, 3, H, D] (+ bias [3, H, D]) -> q/k/v [B, H, S, D], and the
 // biased value is written back into QKV like the reference does
 // (Transpose.cu:41-44).
-__global__ __launch_bounds__(256) void qkv_bias_transpose_f16_kernel(
-    _Float16 *__restrict__ q, _Float16 *__restrict__ k, _Float16 *__restrict__ v,
-    _Float16 *__restrict__ qkv, const _Float16 *__restrict__ bias, int S, int tokens, int H,
-    int D) {
+template <typename T>
+__global__ __launch_bounds__(256) void qkv_bias_transpose_kernel(T *__restrict__ q, T *__restrict__ k,
+                                                                 T *__restrict__ v, T *__restrict__ qkv,
+                                                                 const T *__restrict__ bias, int S, int tokens,
+                                                                 int H, int D) {
   const int dv = D / 8; // vectors per head row
   const size_t total = (size_t)tokens * 3 * H * dv;
   const size_t stride = (size_t)gridDim.x * 256;
-  _Float16 *const dst[3] = {q, k, v};
+  T *const dst[3] = {q, k, v};
   for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += stride) {
     const int d0 = (int)(idx % dv) * 8;
     size_t r = idx / dv;
@@ -95,56 +87,76 @@ __global__ __launch_bounds__(256) void qkv_bias_transpose_f16_kernel(
     const int which = (int)(r % 3);
     const int token = (int)(r / 3);
     const int b = token / S, s = token % S;
-    f16x8 *src = reinterpret_cast<f16x8 *>(qkv + (((size_t)token * 3 + which) * H + head) * D + d0);
-    f16x8 val = *src;
+    u32x4 *src = reinterpret_cast<u32x4 *>(qkv + (((size_t)token * 3 + which) * H + head) * D + d0);
+    u32x4 val = *src;
     if (bias) {
-      const f16x8 bv = *reinterpret_cast<const f16x8 *>(bias + ((size_t)which * H + head) * D + d0);
+      float x[8], bv[8];
+      ElemTraits<T>::unpack(val, x);
+      ElemTraits<T>::unpack(*reinterpret_cast<const u32x4 *>(bias + ((size_t)which * H + head) * D + d0), bv);
 #pragma unroll
-      for (int e = 0; e < 8; e++) val[e] = (_Float16)((float)val[e] + (float)bv[e]);
+      for (int e = 0; e < 8; e++) x[e] += bv[e];
+      val = ElemTraits<T>::pack(x);
       *src = val;
     }
-    *reinterpret_cast<f16x8 *>(dst[which] + (((size_t)b * H + head) * S + s) * D + d0) = val;
+    *reinterpret_cast<u32x4 *>(dst[which] + (((size_t)b * H + head) * S + s) * D + d0) = val;
+  }
+}
+
+} // namespace
+
+namespace {
+
+template <typename T>
+void castFromF32(void *dst, const float *src, size_t size, hipStream_t stream, const char *what) {
+  if (size == 0) return;
+  if (!dst || !src) fail(std::string(what) + ": null pointer");
+  auto *d = static_cast<T *>(dst);
+  size_t done = 0;
+  if (aligned16(dst) && aligned16(src) && size >= 8) {
+    const size_t n8 = size / 8;
+    cast_f32_to_h_vec8_kernel<T><<<dim3(gridFor(n8, 256)), dim3(256), 0, stream>>>(
+        reinterpret_cast<u32x4 *>(d), reinterpret_cast<const f32x4 *>(src), n8);
+    MGPU_CHECK_LAUNCH("cast_f32_to_h_vec8_kernel");
+    done = n8 * 8;
+  }
+  if (done < size) {
+    cast_scalar_kernel<T, float><<<dim3(gridFor(size - done, 256)), dim3(256), 0, stream>>>(d, src, done, size);
+    MGPU_CHECK_LAUNCH("cast_scalar_kernel");
+  }
+}
+
+template <typename T>
+void castToF32(float *dst, const void *src, size_t size, hipStream_t stream, const char *what) {
+  if (size == 0) return;
+  if (!dst || !src) fail(std::string(what) + ": null pointer");
+  auto *s = static_cast<const T *>(src);
+  size_t done = 0;
+  if (aligned16(dst) && aligned16(src) && size >= 8) {
+    const size_t n8 = size / 8;
+    cast_h_to_f32_vec8_kernel<T><<<dim3(gridFor(n8, 256)), dim3(256), 0, stream>>>(
+        reinterpret_cast<f32x4 *>(dst), reinterpret_cast<const u32x4 *>(s), n8);
+    MGPU_CHECK_LAUNCH("cast_h_to_f32_vec8_kernel");
+    done = n8 * 8;
+  }
+  if (done < size) {
+    cast_scalar_kernel<float, T><<<dim3(gridFor(size - done, 256)), dim3(256), 0, stream>>>(dst, s, done, size);
+    MGPU_CHECK_LAUNCH("cast_scalar_kernel");
   }
 }
 
 } // namespace
 
 void castF32ToF16(void *dst, const float *src, size_t size, hipStream_t stream) {
-  if (size == 0) return;
-  if (!dst || !src) fail("castF32ToF16: null pointer");
-  auto *d = static_cast<_Float16 *>(dst);
-  size_t done = 0;
-  if (aligned16(dst) && aligned16(src) && size >= 8) {
-    const size_t n8 = size / 8;
-    cast_f32_to_f16_vec8_kernel<<<dim3(gridFor(n8, 256)), dim3(256), 0, stream>>>(
-        reinterpret_cast<f16x8 *>(d), reinterpret_cast<const f32x4 *>(src), n8);
-    MGPU_CHECK_LAUNCH("cast_f32_to_f16_vec8_kernel");
-    done = n8 * 8;
-  }
-  if (done < size) {
-    cast_scalar_kernel<_Float16, float><<<dim3(gridFor(size - done, 256)), dim3(256), 0, stream>>>(
-        d, src, done, size);
-    MGPU_CHECK_LAUNCH("cast_scalar_kernel");
-  }
+  castFromF32<_Float16>(dst, src, size, stream, "castF32ToF16");
 }
-
 void castF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream) {
-  if (size == 0) return;
-  if (!dst || !src) fail("castF16ToF32: null pointer");
-  auto *s = static_cast<const _Float16 *>(src);
-  size_t done = 0;
-  if (aligned16(dst) && aligned16(src) && size >= 8) {
-    const size_t n8 = size / 8;
-    cast_f16_to_f32_vec8_kernel<<<dim3(gridFor(n8, 256)), dim3(256), 0, stream>>>(
-        reinterpret_cast<f32x4 *>(dst), reinterpret_cast<const f16x8 *>(s), n8);
-    MGPU_CHECK_LAUNCH("cast_f16_to_f32_vec8_kernel");
-    done = n8 * 8;
-  }
-  if (done < size) {
-    cast_scalar_kernel<float, _Float16><<<dim3(gridFor(size - done, 256)), dim3(256), 0, stream>>>(
-        dst, s, done, size);
-    MGPU_CHECK_LAUNCH("cast_scalar_kernel");
-  }
+  castToF32<_Float16>(dst, src, size, stream, "castF16ToF32");
+}
+void castF32ToBF16(void *dst, const float *src, size_t size, hipStream_t stream) {
+  castFromF32<bf16_t>(dst, src, size, stream, "castF32ToBF16");
+}
+void castBF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream) {
+  castToF32<bf16_t>(dst, src, size, stream, "castBF16ToF32");
 }
 
 void fillF16(void *dst, size_t count, float value, hipStream_t stream) {
@@ -160,8 +172,8 @@ void fillI32(int32_t *dst, size_t count, int32_t value, hipStream_t stream) {
   MGPU_CHECK_LAUNCH("fill_kernel");
 }
 
-void addFusedQKVBiasTransposeF16(void *q, void *k, void *v, void *qkv, const void *bias, int B,
-                                 int S, int tokens, int H, int D, hipStream_t stream) {
+void addFusedQKVBiasTranspose(DType dt, void *q, void *k, void *v, void *qkv, const void *bias, int B, int S,
+                              int tokens, int H, int D, hipStream_t stream) {
   if (B < 0 || S < 0 || tokens < 0 || H < 0 || D < 0) fail("addFusedQKVBiasTranspose: negative shape");
   if (tokens == 0 || H == 0 || D == 0) return;
   if (tokens != B * S) fail("addFusedQKVBiasTranspose: token_num must equal batch_size * seq_len");
@@ -170,10 +182,23 @@ void addFusedQKVBiasTransposeF16(void *q, void *k, void *v, void *qkv, const voi
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(qkv) || (bias && !aligned16(bias)))
     fail("addFusedQKVBiasTranspose: pointers must be 16-byte aligned");
   const size_t total = (size_t)tokens * 3 * H * (D / 8);
-  qkv_bias_transpose_f16_kernel<<<dim3(gridFor(total, 256)), dim3(256), 0, stream>>>(
-      static_cast<_Float16 *>(q), static_cast<_Float16 *>(k), static_cast<_Float16 *>(v),
-      static_cast<_Float16 *>(qkv), static_cast<const _Float16 *>(bias), S, tokens, H, D);
-  MGPU_CHECK_LAUNCH("qkv_bias_transpose_f16_kernel");
+  if (dt == DType::F16) {
+    qkv_bias_transpose_kernel<_Float16><<<dim3(gridFor(total, 256)), dim3(256), 0, stream>>>(
+        static_cast<_Float16 *>(q), static_cast<_Float16 *>(k), static_cast<_Float16 *>(v),
+        static_cast<_Float16 *>(qkv), static_cast<const _Float16 *>(bias), S, tokens, H, D);
+  } else if (dt == DType::BF16) {
+    qkv_bias_transpose_kernel<bf16_t><<<dim3(gridFor(total, 256)), dim3(256), 0, stream>>>(
+        static_cast<bf16_t *>(q), static_cast<bf16_t *>(k), static_cast<bf16_t *>(v),
+        static_cast<bf16_t *>(qkv), static_cast<const bf16_t *>(bias), S, tokens, H, D);
+  } else {
+    fail("addFusedQKVBiasTranspose: element type must be fp16 or bf16");
+  }
+  MGPU_CHECK_LAUNCH("qkv_bias_transpose_kernel");
+}
+
+void addFusedQKVBiasTransposeF16(void *q, void *k, void *v, void *qkv, const void *bias, int B,
+                                 int S, int tokens, int H, int D, hipStream_t stream) {
+  addFusedQKVBiasTranspose(DType::F16, q, k, v, qkv, bias, B, S, tokens, H, D, stream);
 }
 
 } // namespace mgpu
@@ -187,13 +212,15 @@ __device__ __forceinline__ float gelu_erf(float x) {
   return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
 }
 
-__global__ __launch_bounds__(256) void gelu_f16_vec8_kernel(f16x8 *__restrict__ data, size_t n8) {
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_h_vec8_kernel(u32x4 *__restrict__ data, size_t n8) {
   const size_t stride = (size_t)gridDim.x * 256;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += stride) {
-    f16x8 v = data[i];
+    float v[8];
+    ElemTraits<T>::unpack(data[i], v);
 #pragma unroll
-    for (int e = 0; e < 8; e++) v[e] = (_Float16)gelu_erf((float)v[e]);
-    data[i] = v;
+    for (int e = 0; e < 8; e++) v[e] = gelu_erf(v[e]);
+    data[i] = ElemTraits<T>::pack(v);
   }
 }
 
@@ -202,27 +229,31 @@ __global__ __launch_bounds__(256) void gelu_scalar_kernel(T *__restrict__ data, 
                                                           size_t n) {
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (size_t i = begin + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
-    data[i] = (T)gelu_erf((float)data[i]);
+    data[i] = ElemTraits<T>::fromFloat(gelu_erf(ElemTraits<T>::toFloat(data[i])));
 }
 
 } // namespace
 
-void geluInPlaceF16(void *data, size_t n, hipStream_t stream) {
+namespace {
+template <typename T> void geluInPlaceH(void *data, size_t n, hipStream_t stream) {
   if (n == 0) return;
-  auto *d = static_cast<_Float16 *>(data);
+  auto *d = static_cast<T *>(data);
   size_t done = 0;
   if (aligned16(data) && n >= 8) {
     const size_t n8 = n / 8;
-    gelu_f16_vec8_kernel<<<dim3(gridFor(n8, 256)), dim3(256), 0, stream>>>(
-        reinterpret_cast<f16x8 *>(d), n8);
-    MGPU_CHECK_LAUNCH("gelu_f16_vec8_kernel");
+    gelu_h_vec8_kernel<T><<<dim3(gridFor(n8, 256)), dim3(256), 0, stream>>>(reinterpret_cast<u32x4 *>(d), n8);
+    MGPU_CHECK_LAUNCH("gelu_h_vec8_kernel");
     done = n8 * 8;
   }
   if (done < n) {
-    gelu_scalar_kernel<_Float16><<<dim3(gridFor(n - done, 256)), dim3(256), 0, stream>>>(d, done, n);
+    gelu_scalar_kernel<T><<<dim3(gridFor(n - done, 256)), dim3(256), 0, stream>>>(d, done, n);
     MGPU_CHECK_LAUNCH("gelu_scalar_kernel");
   }
 }
+} // namespace
+
+void geluInPlaceF16(void *data, size_t n, hipStream_t stream) { geluInPlaceH<_Float16>(data, n, stream); }
+void geluInPlaceBF16(void *data, size_t n, hipStream_t stream) { geluInPlaceH<bf16_t>(data, n, stream); }
 
 void geluInPlaceF32(float *data, size_t n, hipStream_t stream) {
   if (n == 0) return;

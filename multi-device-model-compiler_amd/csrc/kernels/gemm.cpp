@@ -231,10 +231,10 @@ void matmulEx(DType dt, const void *input, const void *weight, const void *bias,
   if (act == ACT_GELU) {
     if (dt == DType::F16)
       geluInPlaceF16(output, (size_t)M * N, stream);
-    else if (dt == DType::F32)
-      geluInPlaceF32(static_cast<float *>(output), (size_t)M * N, stream);
+    else if (dt == DType::BF16)
+      geluInPlaceBF16(output, (size_t)M * N, stream);
     else
-      fail("matmul: GELU epilogue is built for fp16 and fp32 only");
+      geluInPlaceF32(static_cast<float *>(output), (size_t)M * N, stream);
   }
 }
 

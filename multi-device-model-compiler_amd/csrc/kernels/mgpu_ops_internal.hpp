@@ -24,9 +24,13 @@ void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int 
 
 void castF32ToF16(void *dst, const float *src, size_t size, hipStream_t stream);
 void castF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream);
+void castF32ToBF16(void *dst, const float *src, size_t size, hipStream_t stream);
+void castBF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream);
 void fillF16(void *dst, size_t count, float value, hipStream_t stream);
 void fillI32(int32_t *dst, size_t count, int32_t value, hipStream_t stream);
 
+void addFusedQKVBiasTranspose(DType dt, void *q, void *k, void *v, void *qkv, const void *bias, int B, int S,
+                              int tokens, int H, int D, hipStream_t stream);
 void addFusedQKVBiasTransposeF16(void *q, void *k, void *v, void *qkv, const void *bias, int B,
                                  int S, int tokens, int H, int D, hipStream_t stream);
 
@@ -61,6 +65,7 @@ void bertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, cons
                          hipStream_t stream);
 
 void geluInPlaceF16(void *data, size_t n, hipStream_t stream);
+void geluInPlaceBF16(void *data, size_t n, hipStream_t stream);
 void geluInPlaceF32(float *data, size_t n, hipStream_t stream);
 
 } // namespace mgpu

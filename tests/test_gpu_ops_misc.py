@@ -63,6 +63,61 @@ def test_matmul_ex_f16_epilogues(pkg, gpu, oracle, rng, M, K, N):
         assert np.all(np.abs(got - ref) <= f16_tol(ref, k_ulp)), (kw.keys(), np.abs(got - ref).max())
 
 
+def bf16_bits(t):
+    import torch
+    return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("n", [1, 7, 8, 9, 1000, 65537])
+def test_bf16_casts_bit_exact(pkg, gpu, oracle, rng, n):
+    """fp32 <-> bf16: round to nearest even on the upper 16 bits, NaN stays NaN."""
+    f = (rng.standard_normal(n) * np.exp(rng.uniform(-60, 60, n))).astype(np.float32)
+    if n >= 9:
+        f[:9] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, 3.3895e38, 1e-40]
+    h = pkg.cast_f32_to_bf16(to_dev(f, gpu))
+    got, ref = bf16_bits(h), oracle.float_to_bf16(f)
+    nan = np.isnan(f)
+    assert np.array_equal(got[~nan], ref[~nan])
+    assert np.all((got[nan] & 0x7f80) == 0x7f80) and np.all((got[nan] & 0x7f) != 0)
+    back = pkg.cast_bf16_to_f32(h).cpu().numpy()
+    assert np.array_equal(back.view(np.uint32), oracle.bf16_to_float(got).view(np.uint32))
+    # independent pin: the upper half of the fp32 pattern, plus the closed-form rounding
+    u = f[~nan].view(np.uint32).astype(np.uint64)
+    assert np.array_equal(ref[~nan], ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16))
+
+
+def test_qkv_bias_transpose_bf16(pkg, gpu, oracle, rng):
+    import torch
+    B, S, H, D = 2, 37, 3, 64
+    qkv = torch.from_numpy(rng.standard_normal((B, S, 3, H, D)).astype(np.float32)).to(gpu).to(torch.bfloat16)
+    bias = torch.from_numpy(rng.standard_normal((3, H, D)).astype(np.float32)).to(gpu).to(torch.bfloat16)
+    qb, bb = bf16_bits(qkv), bf16_bits(bias)
+    q, k, v = pkg.qkv_bias_transpose(qkv, bias)
+    rq, rk, rv = oracle.qkv_bias_transpose(qb, bb, bf16=True)
+    for got, ref in ((q, rq), (k, rk), (v, rv)):
+        assert np.array_equal(got.float().cpu().numpy(), ref)
+    upd = oracle.float_to_bf16(oracle.bf16_to_float(qb) + oracle.bf16_to_float(bb)[None, None])
+    assert np.array_equal(bf16_bits(qkv), upd)
+
+
+@pytest.mark.parametrize("M,K,N", [(256, 768, 768), (100, 64, 72)])
+def test_matmul_ex_bf16_epilogues(pkg, gpu, oracle, rng, M, K, N):
+    import torch
+    mk = lambda a: torch.from_numpy(a.astype(np.float32)).to(gpu).to(torch.bfloat16)
+    tx, tw = mk(rng.standard_normal((M, K))), mk(rng.standard_normal((K, N)) / np.sqrt(K))
+    tb, tr = mk(rng.standard_normal(N)), mk(rng.standard_normal((M, N)))
+    x, w, b, r = [bf16_bits(t) for t in (tx, tw, tb, tr)]
+    for kw, okw in [(dict(), dict()), (dict(bias=tb), dict(bias=b)),
+                    (dict(bias=tb, act=pkg.ACT_RELU), dict(bias=b, act=oracle.ACT_RELU)),
+                    (dict(bias=tb, act=pkg.ACT_GELU), dict(bias=b, act=oracle.ACT_GELU)),
+                    (dict(bias=tb, residual=tr), dict(bias=b, residual=r))]:
+        got = pkg.matmul_ex(tx, tw, **kw).float().cpu().numpy()
+        ref = oracle.gemm(x, w, bf16=True, **okw)
+        # one bf16 spacing of the result (2^-7 relative); GELU rounds twice
+        k_ulp = 2.5 if kw.get("act") == pkg.ACT_GELU else 1.0
+        tol = k_ulp * 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref), 2.0 ** -14))) - 7) + 4e-3
+        assert np.all(np.abs(got - ref) <= tol), (kw.keys(), np.abs(got - ref).max())
+
 def test_matmul_f32(pkg, gpu, oracle, rng):
     M, K, N = 200, 96, 130
     x = rng.standard_normal((M, K)).astype(np.float32)

@@ -125,3 +125,31 @@ def test_resnet_block_plan(pkg, gpu, tmp_path, oracle):
     r = oracle.conv2d(h, w2, b2, x, (1, 1, 1, 1), relu=True)
     ref = oracle.pool2d(r, (2, 2), stride=(2, 2))
     assert np.all(np.abs(y - ref) <= 4e-3 * (1.0 + np.abs(ref)))
+
+
+def test_bf16_pipeline_cast_matmul_cast(pkg, gpu, tmp_path, oracle, rng):
+    """fp32 in -> bf16 cast -> bf16 GEMM with bias and ReLU -> fp32 out: the
+    bf16 entry points reached through the plan lowering."""
+    M, K, N = 64, 128, 96
+    body = f"""func @main_graph(%x: {M}x{K}xf32, %w: {K}x{N}xf32, %b: {N}xf32) -> (%y: {M}x{N}xf32) {{
+  %xh = device.cast %x : {M}x{K}xbf16
+  %wh = device.cast %w : {K}x{N}xbf16
+  %bh = device.cast %b : {N}xbf16
+  %yh = device.matmul-ex %xh, %wh, %bh, none {{act = "relu"}} : {M}x{N}xbf16
+  %y = device.cast %yh : {M}x{N}xf32
+  return
+}}
+"""
+    plan = tmp_path / "bf16.plan"
+    plan.write_text(body)
+    lower = subprocess.run([os.path.join(pkg.BIN_DIR, "multi-device-plan-lower"), str(plan)], capture_output=True, text=True)
+    assert lower.returncode == 0, lower.stderr
+    for callee in ("mgpuCastF32ToBF16", "mgpuMatmulExBF16", "mgpuCastBF16ToF32"):
+        assert callee in lower.stdout
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    y, _ = run_plan(pkg, plan, [x, w, b], np.float32, (M, N), tmp_path)
+    ref = oracle.gemm(oracle.float_to_bf16(x), oracle.float_to_bf16(w), oracle.float_to_bf16(b), act=oracle.ACT_RELU, bf16=True)
+    tol = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref), 2.0 ** -14))) - 7) + 4e-3
+    assert np.all(np.abs(y - ref) <= tol), np.abs(y - ref).max()
