@@ -2,9 +2,9 @@
 
 Pooling is exact (max) or one fp32 rounding of the window sum (average).  The
 convolution accumulates fp32 products on the matrix cores in an order of its
-own; the bound of 2e-3 (1 + |ref|), checked elementwise, also admits the
-reduced-precision products the reference allows through
-CUDNN_TENSOR_OP_MATH_ALLOW_CONVERSION."""
+own (true fp32 products, unlike the reduced-precision ones the reference
+allows through CUDNN_TENSOR_OP_MATH_ALLOW_CONVERSION): the bound is
+1e-4 (1 + |ref|), checked elementwise."""
 import numpy as np
 import pytest
 
@@ -24,7 +24,7 @@ def conv_case(pkg, gpu, oracle, rng, N, IC, H, W, OC, K, pad, stride, dilation, 
                      pad, stride, dilation, relu).cpu().numpy()
     assert got.shape == ref.shape
     err = np.abs(got - ref)
-    assert np.all(err <= 2e-3 * (1.0 + np.abs(ref))), err.max()
+    assert np.all(err <= 1e-4 * (1.0 + np.abs(ref))), err.max()
     return err.max()
 
 
