@@ -410,6 +410,30 @@ def main():
                                      "frac": round(flop / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
                         "algorithmic_flop": flop})
 
+    if want("conv2d"):
+        # the shape of the reference's End2End conv test: 16x3x256x256 -> 64 channels, 3x3, pad 1
+        N_, IC, H_, W_, OC = 16, 3, 256, 256, 64
+        xc = torch.randn((N_, IC, H_, W_), device=dev, generator=gen)
+        wc = 0.1 * torch.randn((OC, IC, 3, 3), device=dev, generator=gen)
+        bc = torch.randn(OC, device=dev, generator=gen)
+        yc = torch.empty((N_, OC, H_, W_), device=dev)
+
+        def conv(i):
+            lib.mgpuConv2d(xc.data_ptr(), wc.data_ptr(), bc.data_ptr(), yc.data_ptr(), None, N_, IC, H_, W_, OC, 3, 3,
+                           H_, W_, 1, 1, 1, 1, 1, 1, 1, 1, False, False, torch.cuda.current_stream().cuda_stream)
+
+        steps = max(10, K // 10)
+        ms = Timer(torch, use_graph=False).run(conv, steps, 3)
+        check()
+        us = ms * 1e3 / steps
+        nbytes = (xc.numel() + wc.numel() + bc.numel() + yc.numel()) * 4
+        flop = 2.0 * N_ * OC * H_ * W_ * IC * 9
+        kernels.append({"name": "conv2d", "workload": "conv2d fp32 16x3x256x256 -> 64, 3x3 pad 1", "dtype": "f32",
+                        "metric": "us", "value": round(us, 1), "higher_is_better": False,
+                        "roofline": {"bound": "hbm", "achieved": round(nbytes / us / 1e3, 1), "peak": HBM_PEAK_GBS,
+                                     "unit": "GB/s", "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None},
+                        "algorithmic_bytes": nbytes, "algorithmic_flop": flop})
+
     # ---------------- CPU baseline: the oracle on the host cores ---------------
     cpu = None
     if not args.no_cpu:
