@@ -329,7 +329,7 @@ def main():
         del al, bl, cl
 
     # ---------------- fused MHA -------------------------------------------------
-    def fmha_case(name, workload, B, S, H, masked, D=64):
+    def fmha_case(name, workload, B, S, H, masked, D=64, causal=False):
         qkv = (torch.randn((B, S, 3, H, D), device=dev, generator=gen) / 8).half()
         out = torch.empty((B, S, H * D), device=dev, dtype=torch.float16)
         lens = None
@@ -338,20 +338,22 @@ def main():
             lens_cpu = torch.randint(256, 513, (B,), generator=torch.Generator().manual_seed(20244), dtype=torch.int32)
             lens = lens_cpu.to(dev)
             flop_valid = 4.0 * H * D * S * float(lens_cpu.sum())
+        elif causal:
+            flop_valid = 4.0 * B * H * D * (S * (S + 1) / 2)  # query i sees keys 0..i
         else:
             flop_valid = flop
 
         def run(i):
             s = torch.cuda.current_stream().cuda_stream
             lib.mgpuFusedMHAF16(qkv.data_ptr(), lens.data_ptr() if lens is not None else None,
-                                out.data_ptr(), B, S, H, D, D ** -0.5, 0, s)
+                                out.data_ptr(), B, S, H, D, D ** -0.5, int(causal), s)
 
         steps = max(20, K // 4)
         if loops:
             torch.cuda.synchronize()
             ms = loop_ms(loops.mgpuBenchFusedMHAF16(
                 ptrs([qkv]), ptrs([out]), 1, ctypes.c_void_p(lens.data_ptr() if lens is not None else None),
-                B, S, H, D, ctypes.c_float(D ** -0.5), 0, steps, max(3, W // 4), sp))
+                B, S, H, D, ctypes.c_float(D ** -0.5), int(causal), steps, max(3, W // 4), sp))
         else:
             ms = timer.run(run, steps, max(3, W // 4))
         check()
@@ -365,7 +367,7 @@ def main():
                               "traffic": TRAFFIC_BYTES.get(name)},
                  "algorithmic_flop": flop_valid, "algorithmic_bytes": nbytes,
                  "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
-        if masked:
+        if masked or causal:
             entry["dense_flop"] = flop
         kernels.append(entry)
 
@@ -376,6 +378,10 @@ def main():
                   8, 512, 16, True)
     if want("fmha_b32_s512"):
         fmha_case("fmha_b32_s512", "fused MHA fp16 b32 s512 h12 d64 [roofline target shape]", 32, 512, 12, False)
+
+    if want("fmha_b32_s512_causal"):
+        fmha_case("fmha_b32_s512_causal", "fused MHA fp16 b32 s512 h12 d64, causal (the reference layer's mask)",
+                  32, 512, 12, False, causal=True)
 
     if want("fmha_d128_b32_s512"):
         fmha_case("fmha_d128_b32_s512", "fused MHA fp16 b32 s512 h8 d128 [the reference layer's head geometry]",

@@ -156,10 +156,10 @@ __device__ __forceinline__ float halves_sum(float v) {
 }
 
 template <typename T, int D, int NQ, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void fmha_fwd_kernel(const uint16_t *__restrict__ qkv,
+__global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_kernel(const uint16_t *__restrict__ qkv,
                                                               const int32_t *__restrict__ seqlens,
                                                               uint16_t *__restrict__ out, int S, int H,
-                                                              int nQB, float scale_log2e) {
+                                                              int nQB, float scale_log2e, int pairItems) {
   using M = Mma<T>;
   using v8 = typename M::v8;
   using v4 = typename M::v4;
@@ -178,8 +178,16 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_kernel(const uint16_t *__rest
   const int nblk = gridDim.x;
   const int bid = blockIdx.x;
   const int wid = (nblk % 8 == 0) ? (bid % 8) * (nblk / 8) + bid / 8 : bid;
-  const int qb = wid % nQB;
-  const int bh = wid / nQB;
+  // Causal: query block i of a (batch, head) needs i + 1 of the nQB key
+  // ranges.  When the launcher asks for it (pairItems), block i and block
+  // nQB - 1 - i are given to one work item, the long one first, so that every
+  // work item carries the same number of tiles; left alone, the items with the
+  // last query blocks run as long as without the mask while the others sit idle.
+  constexpr bool kCanPair = CAUSAL && D == 64; // elsewhere the second pass is compiled out
+  const bool paired = kCanPair && pairItems;
+  const int nItems = paired ? (nQB + 1) / 2 : nQB; // work items per (batch, head)
+  const int item = wid % nItems;
+  const int bh = wid / nItems;
   const int h = bh % H;
   const int b = bh / H;
 
@@ -194,12 +202,16 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_kernel(const uint16_t *__rest
     kvlen = seqlens[b];
     kvlen = kvlen < 0 ? 0 : (kvlen > S ? S : kvlen);
   }
-  const int q0 = qb * BM + wave * (NQ * 32); // first query of this wavefront
   const uint32_t tokBytes = (uint32_t)3 * H * kD * 2; // bytes per token row
   const char *qbase = reinterpret_cast<const char *>(qkv) + ((size_t)b * S * 3 * H + h) * kD * 2;
   const char *kbase = qbase + (size_t)H * kD * 2;
   const char *vbase = qbase + (size_t)2 * H * kD * 2;
 
+  const int nParts = (kCanPair && paired && item != nQB - 1 - item) ? 2 : 1;
+#pragma clang loop unroll(disable)
+  for (int part = 0; part < nParts; part++) {
+  const int qb = paired ? (part == 0 ? nQB - 1 - item : item) : item;
+  const int q0 = qb * BM + wave * (NQ * 32); // first query of this wavefront
   int kend = kvlen;
   if (CAUSAL) {
     int lastq = qb * BM + BM - 1;
@@ -471,6 +483,22 @@ __global__ __launch_bounds__(256, 2) void fmha_fwd_kernel(const uint16_t *__rest
           val, reinterpret_cast<u32x4 *>(out + ((size_t)b * S + query) * H * kD + (size_t)h * kD + cidx * 8));
     }
   }
+  // the next part's tiles land in the ring the staging area sits in
+  if (part + 1 < nParts) __syncthreads();
+  } // part
+}
+
+// Compute units of the current device (asked once per device).
+int deviceComputeUnits() {
+  static int cached[64]; // 0 = not asked yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int v = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+  if (v == 0) {
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    __atomic_store_n(&cached[dev], v, __ATOMIC_RELAXED);
+  }
+  return v;
 }
 
 template <typename T, int D, int NQ>
@@ -478,15 +506,19 @@ void launch(const void *qkv, const int32_t *seqlens, void *out, int B, int S, in
             bool causal, hipStream_t stream) {
   constexpr int BM = 128 * NQ;
   const int nQB = (S + BM - 1) / BM;
-  const int64_t blocks = (int64_t)B * H * nQB;
+  // Causal query blocks go in pairs of equal total work when the head dimension
+  // is 64 (at 128 the second pass does not fit the register budget of three
+  // wavefronts per SIMD) and the halved grid still gives every CU two blocks.
+  const bool pair = causal && D == 64 && (int64_t)B * H * ((nQB + 1) / 2) >= 2 * (int64_t)deviceComputeUnits();
+  const int64_t blocks = (int64_t)B * H * (pair ? (nQB + 1) / 2 : nQB);
   if (blocks > 0x7fffffffLL) fail("fusedMHA: problem too large for one launch");
   const float c = scale * 1.44269504088896340736f;
   const auto *in = static_cast<const uint16_t *>(qkv);
   auto *o = static_cast<uint16_t *>(out);
   if (causal)
-    fmha_fwd_kernel<T, D, NQ, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, o, S, H, nQB, c);
+    fmha_fwd_kernel<T, D, NQ, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, o, S, H, nQB, c, pair ? 1 : 0);
   else
-    fmha_fwd_kernel<T, D, NQ, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, o, S, H, nQB, c);
+    fmha_fwd_kernel<T, D, NQ, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, o, S, H, nQB, c, pair ? 1 : 0);
   MGPU_CHECK_LAUNCH("fmha_fwd_kernel");
 }
 
