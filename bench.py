@@ -416,6 +416,36 @@ def main():
                                      "frac": round(flop / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
                         "algorithmic_flop": flop})
 
+    if want("decoding_layer"):
+        # mgpuLLMDecodingContextLayer at the geometry of the reference's own benchmark layer
+        # (benchmark/PyTorch/Models/LLM.py: d_model 2048, 16 heads of 128, feed-forward 2048, causal, ReLU)
+        B, S, d, ffn, H = 8, 512, 2048, 2048, 16
+
+        def f(*shape, s=0.02):
+            return s * torch.randn(shape, device=dev, generator=gen)
+
+        x = torch.randn((B, S, d), device=dev, generator=gen)
+        P = [f(d, 3 * d), f(d, d), f(d), f(d, ffn), f(ffn), f(ffn, d), f(d)]
+        out = torch.empty_like(x)
+
+        def dec(i):
+            lib.mgpuLLMDecodingContextLayer(x.data_ptr(), *[p.data_ptr() for p in P], out.data_ptr(), B, S, d, ffn, H,
+                                            True, True, True, torch.cuda.current_stream().cuda_stream)
+
+        steps = max(10, K // 10)
+        ms = Timer(torch, use_graph=False).run(dec, steps, 3)
+        check()
+        us = ms * 1e3 / steps
+        flop = 2.0 * B * S * d * (3 * d + d + 2 * ffn) + 4.0 * B * H * (d // H) * (S * (S + 1) / 2)
+        kernels.append({"name": "decoding_layer",
+                        "workload": "mgpuLLMDecodingContextLayer fp32 in/out (8,512,2048), 16 heads of 128, ffn 2048, "
+                                    "causal, ReLU; fp32 weights cast to fp16 on every call, as in the reference",
+                        "dtype": "f16", "metric": "us", "value": round(us, 1), "higher_is_better": False,
+                        "roofline": {"bound": "mfma", "achieved": round(flop / us / 1e6, 1),
+                                     "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                     "frac": round(flop / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+                        "algorithmic_flop": flop})
+
     if want("conv2d"):
         # the shape of the reference's End2End conv test: 16x3x256x256 -> 64 channels, 3x3, pad 1
         N_, IC, H_, W_, OC = 16, 3, 256, 256, 64
