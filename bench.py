@@ -318,6 +318,21 @@ def main():
         kernels.append(hbm_entry("layernorm_f32_large", f"LayerNorm fp32 ({mL},{n})", "f32",
                                  2 * mL * n * 4 + 2 * n * 4, ms, 20))
         del xl, yl
+    if want("layernorm_f32_wide") and loops:
+        # a wide row (an LLM hidden size): one 256-thread block holds the row in registers
+        mW, nW = 4096, 8192
+        nsW = rotating_sets(2 * mW * nW * 4)
+        xw = [torch.randn((mW, nW), device=dev, generator=gen) for _ in range(nsW)]
+        yw = [torch.empty((mW, nW), device=dev) for _ in range(nsW)]
+        gw = 1 + 0.02 * torch.randn(nW, device=dev, generator=gen)
+        bw = 0.02 * torch.randn(nW, device=dev, generator=gen)
+        torch.cuda.synchronize()
+        ms = loop_ms(loops.mgpuBenchLayerNormF32(ptrs(xw), ptrs(yw), nsW, ctypes.c_void_p(gw.data_ptr()),
+                                                 ctypes.c_void_p(bw.data_ptr()), ctypes.c_float(1e-5), mW, nW, 50, 5, sp))
+        check()
+        kernels.append(hbm_entry("layernorm_f32_wide", f"LayerNorm fp32 ({mW},{nW})", "f32",
+                                 2 * mW * nW * 4 + 2 * nW * 4, ms, 50))
+        del xw, yw
     if want("add_f32_large") and loops:
         nl = 1 << 28
         al, bl = torch.rand(nl, device=dev, generator=gen), torch.rand(nl, device=dev, generator=gen)

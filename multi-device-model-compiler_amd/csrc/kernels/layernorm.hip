@@ -8,8 +8,10 @@
 //   (mean, then centred sum of squares) reduction over registers and DPP /
 //   lane-exchange sums, one 128-bit non-temporal store per vector (plain loads
 //   + non-temporal stores measured fastest on MI355X).  One pass over HBM.
-// Rows wider than a wavefront can hold, rows whose length is not a multiple of
-// the vector width, and unaligned pointers take a block-per-row kernel.
+// Rows wider than a wavefront can hold live in the registers of a whole block
+// (layernorm_block_kernel); rows whose length is not a multiple of the vector
+// width, rows beyond 256 x 16 vectors and unaligned pointers take the general
+// block-per-row kernel.
 #include "common.hpp"
 #include "mgpu_ops_internal.hpp"
 #include "types.hpp"
@@ -117,6 +119,105 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
           // The sum is stored rounded to T and the normalised value is taken
           // from that rounded sum, while mean and variance came from the
           // un-rounded fp32 sums (reference dataflow, LayerNorm.cu:203-233).
+          const u32x4 packed = Tr::pack(x[k]);
+          __builtin_nontemporal_store(packed, sv + v);
+          Tr::unpack(packed, x[k]);
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; e++) y[e] = (x[k][e] - mean) * rstd * g[e] + b[e];
+        __builtin_nontemporal_store(Tr::pack(y), yv + v);
+      }
+    }
+  }
+}
+
+// Rows too wide for one wavefront's registers: the same scheme with a whole
+// 256-thread block per row (up to 256 x 16 vectors: 16384 fp32 or 32768
+// 16-bit elements), the two reductions finished across the 4 wavefronts
+// through LDS.  Still one pass over HBM.  gamma and beta are read where they
+// are used: holding them would double the registers of a wide row.
+template <typename T, int VPL, bool RESIDUAL, bool FULL>
+__global__ __launch_bounds__(256) void layernorm_block_kernel(
+    const T *__restrict__ input, const T *__restrict__ residual, const T *__restrict__ gamma,
+    const T *__restrict__ beta, T *__restrict__ sumOut, T *__restrict__ normed, float eps, int m,
+    int n) {
+  using Tr = ElemTraits<T>;
+  constexpr int VEC = Tr::kVec;
+  __shared__ float partial[2][4];
+  const int t = threadIdx.x, wave = t / 64;
+  const int nvec = n / VEC;
+  const float inv_n = 1.0f / (float)n;
+  const u32x4 *gv = reinterpret_cast<const u32x4 *>(gamma);
+  const u32x4 *bv = reinterpret_cast<const u32x4 *>(beta);
+
+  for (int row = blockIdx.x; row < m; row += gridDim.x) {
+    const u32x4 *xv = reinterpret_cast<const u32x4 *>(input + (size_t)row * n);
+    const u32x4 *rv = RESIDUAL ? reinterpret_cast<const u32x4 *>(residual + (size_t)row * n) : nullptr;
+    u32x4 raw[VPL], rawr[VPL];
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = t + k * 256;
+      if (FULL || v < nvec) {
+        raw[k] = xv[v];
+        if (RESIDUAL) rawr[k] = rv[v];
+      }
+    }
+    float x[VPL][VEC];
+    float sum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = t + k * 256;
+      if (FULL || v < nvec) {
+        Tr::unpack(raw[k], x[k]);
+        if (RESIDUAL) {
+          float r[VEC];
+          Tr::unpack(rawr[k], r);
+#pragma unroll
+          for (int e = 0; e < VEC; e++) x[k][e] += r[e];
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; e++) sum += x[k][e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) x[k][e] = 0.0f;
+      }
+    }
+    // Two barriers per row are enough: a wavefront that writes partial[0] for
+    // the next row has passed the second barrier of this one, i.e. every
+    // wavefront has read partial[0]; the same holds for partial[1] one barrier on.
+    sum = group_sum<64>(sum);
+    if (t % 64 == 0) partial[0][wave] = sum;
+    __syncthreads();
+    const float mean = (partial[0][0] + partial[0][1] + partial[0][2] + partial[0][3]) * inv_n;
+
+    float sq = 0.0f;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = t + k * 256;
+      if (FULL || v < nvec) {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+          const float d = x[k][e] - mean;
+          sq += d * d;
+        }
+      }
+    }
+    sq = group_sum<64>(sq);
+    if (t % 64 == 0) partial[1][wave] = sq;
+    __syncthreads();
+    const float var = (partial[1][0] + partial[1][1] + partial[1][2] + partial[1][3]) * inv_n;
+    const float rstd = 1.0f / sqrtf(var + eps);
+
+    u32x4 *yv = reinterpret_cast<u32x4 *>(normed + (size_t)row * n);
+    u32x4 *sv = RESIDUAL ? reinterpret_cast<u32x4 *>(sumOut + (size_t)row * n) : nullptr;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = t + k * 256;
+      if (FULL || v < nvec) {
+        float g[VEC], b[VEC], y[VEC];
+        Tr::unpack(gv[v], g);
+        Tr::unpack(bv[v], b);
+        if (RESIDUAL) { // rounded sum out, normalised value from the rounded sum (see above)
           const u32x4 packed = Tr::pack(x[k]);
           __builtin_nontemporal_store(packed, sv + v);
           Tr::unpack(packed, x[k]);
@@ -242,6 +343,26 @@ void layerNormTyped(const T *input, const T *residual, const T *gamma, const T *
   int64_t blocks = m;
   const int64_t cap = kMaxStreamBlocks;
   if (blocks > cap) blocks = cap;
+  if (vectorOk && nvec <= 256 * 16) {
+    // smallest of 4 / 8 / 12 / 16 vectors per thread that holds the row
+    const int vpl = nvec <= 256 * 4 ? 4 : nvec <= 256 * 8 ? 8 : nvec <= 256 * 12 ? 12 : 16;
+    const bool full = nvec == 256 * vpl;
+#define MGPU_LN_BLOCK(V, F)                                                                      \
+  layernorm_block_kernel<T, V, RESIDUAL, F><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(   \
+      input, residual, gamma, beta, sumOut, normed, eps, m, n)
+    if (vpl == 4) {
+      if (full) MGPU_LN_BLOCK(4, true); else MGPU_LN_BLOCK(4, false);
+    } else if (vpl == 8) {
+      if (full) MGPU_LN_BLOCK(8, true); else MGPU_LN_BLOCK(8, false);
+    } else if (vpl == 12) {
+      if (full) MGPU_LN_BLOCK(12, true); else MGPU_LN_BLOCK(12, false);
+    } else {
+      if (full) MGPU_LN_BLOCK(16, true); else MGPU_LN_BLOCK(16, false);
+    }
+#undef MGPU_LN_BLOCK
+    MGPU_CHECK_LAUNCH("layernorm_block_kernel");
+    return;
+  }
   layernorm_general_kernel<T, RESIDUAL><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
       input, residual, gamma, beta, sumOut, normed, eps, m, n);
   MGPU_CHECK_LAUNCH("layernorm_general_kernel");

@@ -56,7 +56,10 @@ def test_layernorm_config1_fp16_full_size(pkg, gpu, oracle):
 # very wide rows
 @pytest.mark.parametrize("m,n", [(1, 4), (3, 64), (5, 100), (7, 256), (9, 260), (4, 512), (6, 768),
                                  (5, 1000), (3, 1024), (2, 2048), (2, 2052), (3, 4096), (2, 8200),
-                                 (5, 1), (4, 2), (3, 6), (3, 7), (2, 770), (1, 12289), (1000, 96)])
+                                 (5, 1), (4, 2), (3, 6), (3, 7), (2, 770), (1, 12289), (1000, 96),
+                                 # the block-per-row register kernel: 4 / 8 / 16 vectors per thread, full and ragged
+                                 (5, 3072), (7, 4096), (3, 5000), (6, 8192), (4, 12288), (5, 16384), (2, 16388),
+                                 (600, 4096)])
 def test_layernorm_fp32_shapes(pkg, gpu, oracle, rng, m, n):
     x = (rng.standard_normal((m, n)) * 2 + 0.5).astype(np.float32)
     g = rng.standard_normal(n).astype(np.float32)
@@ -68,7 +71,8 @@ def test_layernorm_fp32_shapes(pkg, gpu, oracle, rng, m, n):
 
 
 @pytest.mark.parametrize("m,n", [(3, 8), (4, 128), (5, 768), (2, 1000), (3, 1024), (2, 4096), (3, 8192),
-                                 (2, 9), (3, 770), (2, 20000)])
+                                 (2, 9), (3, 770), (2, 20000), (5, 16384), (3, 24576), (4, 32768), (2, 32776),
+                                 (300, 8192)])
 def test_layernorm_fp16_shapes(pkg, gpu, oracle, rng, m, n):
     x = rng.standard_normal((m, n)).astype(np.float16)
     g = rng.standard_normal(n).astype(np.float16)
@@ -91,7 +95,7 @@ def test_layernorm_bf16(pkg, gpu, oracle, rng):
 
 
 def test_add_residual_layernorm_fp16(pkg, gpu, oracle, rng):
-    for m, n in [(4096, 768), (5, 1000), (3, 77)]:
+    for m, n in [(4096, 768), (5, 1000), (3, 77), (64, 8192), (5, 12288), (3, 32768)]:
         a = rng.standard_normal((m, n)).astype(np.float16)
         r = rng.standard_normal((m, n)).astype(np.float16)
         g, b = params(rng, n, np.float16)
@@ -101,10 +105,11 @@ def test_add_residual_layernorm_fp16(pkg, gpu, oracle, rng):
         assert np.all(np.abs(y.cpu().numpy().astype(np.float32) - ry) <= ulp16(ry))
 
 
-def test_add_residual_layernorm_fp32(pkg, gpu, oracle, rng):
-    a = rng.standard_normal((300, 768)).astype(np.float32)
-    r = rng.standard_normal((300, 768)).astype(np.float32)
-    g, b = params(rng, 768)
+@pytest.mark.parametrize("m,n", [(300, 768), (33, 4096), (5, 6000), (4, 16384)])
+def test_add_residual_layernorm_fp32(pkg, gpu, oracle, rng, m, n):
+    a = rng.standard_normal((m, n)).astype(np.float32)
+    r = rng.standard_normal((m, n)).astype(np.float32)
+    g, b = params(rng, n)
     s, y = pkg.add_residual_layer_norm(to_dev(a, gpu), to_dev(r, gpu), to_dev(g, gpu), to_dev(b, gpu))
     rs, ry = oracle.add_residual_layernorm(a, r, g, b)
     assert np.array_equal(s.cpu().numpy(), rs)
