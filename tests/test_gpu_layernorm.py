@@ -84,7 +84,7 @@ def test_layernorm_fp16_shapes(pkg, gpu, oracle, rng, m, n):
 
 def test_layernorm_bf16(pkg, gpu, oracle, rng):
     import torch
-    for m, n in [(64, 768), (3, 1000), (2, 333)]:
+    for m, n in [(64, 768), (3, 1000), (2, 333), (5, 8192), (3, 12288), (2, 32768)]:
         xf = rng.standard_normal((m, n)).astype(np.float32)
         gf, bf = params(rng, n)
         x, g, b = [torch.from_numpy(t).to(gpu).to(torch.bfloat16) for t in (xf, gf, bf)]
