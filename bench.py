@@ -55,6 +55,7 @@ TRAFFIC_BYTES = {
     "fmha_b32_s512": 100_780_000,
     "fmha_d128_b32_s512": 134_300_000,
 }
+# (fmha_b32_s512_causal, fmha_d128_b4_s2048, conv2d and the layers have no counter run behind them: traffic null)
 
 
 def parse_args():
@@ -401,6 +402,10 @@ def main():
     if want("fmha_d128_b32_s512"):
         fmha_case("fmha_d128_b32_s512", "fused MHA fp16 b32 s512 h8 d128 [the reference layer's head geometry]",
                   32, 512, 8, False, D=128)
+
+    if want("fmha_d128_b4_s2048"):
+        fmha_case("fmha_d128_b4_s2048", "fused MHA fp16 b4 s2048 h32 d128 [long sequences, the reference layer's head size]",
+                  4, 2048, 32, False, D=128)
 
     # ---------------- BERT-base encoder layer ----------------------------------
     if want("bert_layer"):
