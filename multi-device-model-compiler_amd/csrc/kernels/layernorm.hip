@@ -135,96 +135,125 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
 // 256-thread block per row (up to 256 x 16 vectors: 16384 fp32 or 32768
 // 16-bit elements), the two reductions finished across the 4 wavefronts
 // through LDS.  Still one pass over HBM.  gamma and beta are read where they
-// are used: holding them would double the registers of a wide row.
-template <typename T, int VPL, bool RESIDUAL, bool FULL>
+// are used (holding them would double the registers of a wide row); with
+// ROWS = 2 a block works on two rows at a time, which halves that re-reading
+// and the barriers per row and keeps more loads in flight.
+template <typename T, int VPL, int ROWS, bool RESIDUAL, bool FULL>
 __global__ __launch_bounds__(256) void layernorm_block_kernel(
     const T *__restrict__ input, const T *__restrict__ residual, const T *__restrict__ gamma,
     const T *__restrict__ beta, T *__restrict__ sumOut, T *__restrict__ normed, float eps, int m,
     int n) {
   using Tr = ElemTraits<T>;
   constexpr int VEC = Tr::kVec;
-  __shared__ float partial[2][4];
+  __shared__ float partial[2][ROWS][4];
   const int t = threadIdx.x, wave = t / 64;
   const int nvec = n / VEC;
   const float inv_n = 1.0f / (float)n;
   const u32x4 *gv = reinterpret_cast<const u32x4 *>(gamma);
   const u32x4 *bv = reinterpret_cast<const u32x4 *>(beta);
 
-  for (int row = blockIdx.x; row < m; row += gridDim.x) {
-    const u32x4 *xv = reinterpret_cast<const u32x4 *>(input + (size_t)row * n);
-    const u32x4 *rv = RESIDUAL ? reinterpret_cast<const u32x4 *>(residual + (size_t)row * n) : nullptr;
-    u32x4 raw[VPL], rawr[VPL];
+  for (int row0 = blockIdx.x * ROWS; row0 < m; row0 += gridDim.x * ROWS) {
+    float x[ROWS][VPL][VEC];
+    float sum[ROWS];
+    {
+      u32x4 raw[ROWS][VPL], rawr[ROWS][VPL];
 #pragma unroll
-    for (int k = 0; k < VPL; k++) {
-      const int v = t + k * 256;
-      if (FULL || v < nvec) {
-        raw[k] = xv[v];
-        if (RESIDUAL) rawr[k] = rv[v];
-      }
-    }
-    float x[VPL][VEC];
-    float sum = 0.0f;
+      for (int r = 0; r < ROWS; r++) {
+        // a row past the end re-reads the last row; its results are not stored
+        const int row = row0 + r < m ? row0 + r : m - 1;
+        const u32x4 *xv = reinterpret_cast<const u32x4 *>(input + (size_t)row * n);
+        const u32x4 *rv = RESIDUAL ? reinterpret_cast<const u32x4 *>(residual + (size_t)row * n) : nullptr;
 #pragma unroll
-    for (int k = 0; k < VPL; k++) {
-      const int v = t + k * 256;
-      if (FULL || v < nvec) {
-        Tr::unpack(raw[k], x[k]);
-        if (RESIDUAL) {
-          float r[VEC];
-          Tr::unpack(rawr[k], r);
-#pragma unroll
-          for (int e = 0; e < VEC; e++) x[k][e] += r[e];
+        for (int k = 0; k < VPL; k++) {
+          const int v = t + k * 256;
+          if (FULL || v < nvec) {
+            raw[r][k] = xv[v];
+            if (RESIDUAL) rawr[r][k] = rv[v];
+          }
         }
-#pragma unroll
-        for (int e = 0; e < VEC; e++) sum += x[k][e];
-      } else {
-#pragma unroll
-        for (int e = 0; e < VEC; e++) x[k][e] = 0.0f;
       }
-    }
-    // Two barriers per row are enough: a wavefront that writes partial[0] for
-    // the next row has passed the second barrier of this one, i.e. every
-    // wavefront has read partial[0]; the same holds for partial[1] one barrier on.
-    sum = group_sum<64>(sum);
-    if (t % 64 == 0) partial[0][wave] = sum;
-    __syncthreads();
-    const float mean = (partial[0][0] + partial[0][1] + partial[0][2] + partial[0][3]) * inv_n;
-
-    float sq = 0.0f;
 #pragma unroll
-    for (int k = 0; k < VPL; k++) {
-      const int v = t + k * 256;
-      if (FULL || v < nvec) {
+      for (int r = 0; r < ROWS; r++) {
+        sum[r] = 0.0f;
 #pragma unroll
-        for (int e = 0; e < VEC; e++) {
-          const float d = x[k][e] - mean;
-          sq += d * d;
+        for (int k = 0; k < VPL; k++) {
+          const int v = t + k * 256;
+          if (FULL || v < nvec) {
+            Tr::unpack(raw[r][k], x[r][k]);
+            if (RESIDUAL) {
+              float rr[VEC];
+              Tr::unpack(rawr[r][k], rr);
+#pragma unroll
+              for (int e = 0; e < VEC; e++) x[r][k][e] += rr[e];
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; e++) sum[r] += x[r][k][e];
+          } else {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) x[r][k][e] = 0.0f;
+          }
         }
       }
     }
-    sq = group_sum<64>(sq);
-    if (t % 64 == 0) partial[1][wave] = sq;
+    // Two barriers per iteration are enough: a wavefront that writes
+    // partial[0] for the next rows has passed the second barrier of this
+    // iteration, i.e. every wavefront has read partial[0]; the same holds for
+    // partial[1] one barrier on.
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+      const float s = group_sum<64>(sum[r]);
+      if (t % 64 == 0) partial[0][r][wave] = s;
+    }
     __syncthreads();
-    const float var = (partial[1][0] + partial[1][1] + partial[1][2] + partial[1][3]) * inv_n;
-    const float rstd = 1.0f / sqrtf(var + eps);
+    float mean[ROWS], sq[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+      mean[r] = (partial[0][r][0] + partial[0][r][1] + partial[0][r][2] + partial[0][r][3]) * inv_n;
+      sq[r] = 0.0f;
+#pragma unroll
+      for (int k = 0; k < VPL; k++) {
+        const int v = t + k * 256;
+        if (FULL || v < nvec) {
+#pragma unroll
+          for (int e = 0; e < VEC; e++) {
+            const float d = x[r][k][e] - mean[r];
+            sq[r] += d * d;
+          }
+        }
+      }
+      const float s = group_sum<64>(sq[r]);
+      if (t % 64 == 0) partial[1][r][wave] = s;
+    }
+    __syncthreads();
+    float rstd[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+      const float var = (partial[1][r][0] + partial[1][r][1] + partial[1][r][2] + partial[1][r][3]) * inv_n;
+      rstd[r] = 1.0f / sqrtf(var + eps);
+    }
 
-    u32x4 *yv = reinterpret_cast<u32x4 *>(normed + (size_t)row * n);
-    u32x4 *sv = RESIDUAL ? reinterpret_cast<u32x4 *>(sumOut + (size_t)row * n) : nullptr;
 #pragma unroll
     for (int k = 0; k < VPL; k++) {
       const int v = t + k * 256;
       if (FULL || v < nvec) {
-        float g[VEC], b[VEC], y[VEC];
+        float g[VEC], b[VEC];
         Tr::unpack(gv[v], g);
         Tr::unpack(bv[v], b);
-        if (RESIDUAL) { // rounded sum out, normalised value from the rounded sum (see above)
-          const u32x4 packed = Tr::pack(x[k]);
-          __builtin_nontemporal_store(packed, sv + v);
-          Tr::unpack(packed, x[k]);
-        }
 #pragma unroll
-        for (int e = 0; e < VEC; e++) y[e] = (x[k][e] - mean) * rstd * g[e] + b[e];
-        __builtin_nontemporal_store(Tr::pack(y), yv + v);
+        for (int r = 0; r < ROWS; r++) {
+          if (row0 + r >= m) continue;
+          u32x4 *yv = reinterpret_cast<u32x4 *>(normed + (size_t)(row0 + r) * n);
+          float y[VEC];
+          if (RESIDUAL) { // rounded sum out, normalised value from the rounded sum (see above)
+            u32x4 *sv = reinterpret_cast<u32x4 *>(sumOut + (size_t)(row0 + r) * n);
+            const u32x4 packed = Tr::pack(x[r][k]);
+            __builtin_nontemporal_store(packed, sv + v);
+            Tr::unpack(packed, x[r][k]);
+          }
+#pragma unroll
+          for (int e = 0; e < VEC; e++) y[e] = (x[r][k][e] - mean[r]) * rstd[r] * g[e] + b[e];
+          __builtin_nontemporal_store(Tr::pack(y), yv + v);
+        }
       }
     }
   }
@@ -344,20 +373,28 @@ void layerNormTyped(const T *input, const T *residual, const T *gamma, const T *
   const int64_t cap = kMaxStreamBlocks;
   if (blocks > cap) blocks = cap;
   if (vectorOk && nvec <= 256 * 16) {
-    // smallest of 4 / 8 / 12 / 16 vectors per thread that holds the row
+    // smallest of 4 / 8 / 12 / 16 vectors per thread that holds the row; two
+    // rows per block at a time while they fit the registers of three or four
+    // blocks per CU (fp32 up to 8 vectors, 16-bit types up to 4)
     const int vpl = nvec <= 256 * 4 ? 4 : nvec <= 256 * 8 ? 8 : nvec <= 256 * 12 ? 12 : 16;
     const bool full = nvec == 256 * vpl;
-#define MGPU_LN_BLOCK(V, F)                                                                      \
-  layernorm_block_kernel<T, V, RESIDUAL, F><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(   \
+    const bool pairRows = m >= 2 && vpl * ElemTraits<T>::kVec <= 32;
+    if (pairRows) blocks = (blocks + 1) / 2;
+#define MGPU_LN_BLOCK(V, R, F)                                                                    \
+  layernorm_block_kernel<T, V, R, RESIDUAL, F><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>( \
       input, residual, gamma, beta, sumOut, normed, eps, m, n)
-    if (vpl == 4) {
-      if (full) MGPU_LN_BLOCK(4, true); else MGPU_LN_BLOCK(4, false);
+    if (vpl == 4 && pairRows) {
+      if (full) MGPU_LN_BLOCK(4, 2, true); else MGPU_LN_BLOCK(4, 2, false);
+    } else if (vpl == 4) {
+      if (full) MGPU_LN_BLOCK(4, 1, true); else MGPU_LN_BLOCK(4, 1, false);
+    } else if (vpl == 8 && pairRows) {
+      if (full) MGPU_LN_BLOCK(8, 2, true); else MGPU_LN_BLOCK(8, 2, false);
     } else if (vpl == 8) {
-      if (full) MGPU_LN_BLOCK(8, true); else MGPU_LN_BLOCK(8, false);
+      if (full) MGPU_LN_BLOCK(8, 1, true); else MGPU_LN_BLOCK(8, 1, false);
     } else if (vpl == 12) {
-      if (full) MGPU_LN_BLOCK(12, true); else MGPU_LN_BLOCK(12, false);
+      if (full) MGPU_LN_BLOCK(12, 1, true); else MGPU_LN_BLOCK(12, 1, false);
     } else {
-      if (full) MGPU_LN_BLOCK(16, true); else MGPU_LN_BLOCK(16, false);
+      if (full) MGPU_LN_BLOCK(16, 1, true); else MGPU_LN_BLOCK(16, 1, false);
     }
 #undef MGPU_LN_BLOCK
     MGPU_CHECK_LAUNCH("layernorm_block_kernel");
