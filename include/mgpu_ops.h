@@ -150,6 +150,17 @@ void mgpuMatmulExBF16(void *input, void *weight, void *bias, void *output, void 
                       int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
                       int32_t hasResidual, mgpuStream_t stream);
 
+/* The hand-written MFMA kernel that serves mgpuMatmulExF16 / BF16 where it is
+ * the faster path, callable by itself (no counterpart in the reference):
+ * same arguments; M and N multiples of 128, K a multiple of 32, operands
+ * 16-byte aligned, anything else is an error. */
+void mgpuGemmMfmaF16(void *input, void *weight, void *bias, void *output, void *residual,
+                     int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
+                     int32_t hasResidual, mgpuStream_t stream);
+void mgpuGemmMfmaBF16(void *input, void *weight, void *bias, void *output, void *residual,
+                      int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
+                      int32_t hasResidual, mgpuStream_t stream);
+
 /* ---- transformer layers ----------------------------------------------- */
 /* Pre-LN layer, fp32 in/out, fp16 compute; same signature as the reference
  * (Ops.h:43-48; lib/Kernels/GPU/LLM.cu:26-159). */

@@ -67,6 +67,8 @@ OPS_SIGNATURES = {
     "mgpuPool2d": (None, [_c_void_p] * 2 + [_c_int64] * 15 + [_c_void_p]),
     "mgpuMatmulExF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuMatmulExBF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
+    "mgpuGemmMfmaF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
+    "mgpuGemmMfmaBF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuMatmulExF32": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuLLMDecodingContextLayer": (None, [_c_void_p] * 9 + [_c_int64] * 5 + [ctypes.c_bool] * 3 + [_c_void_p]),
     "mgpuBertEncoderLayerF16": (None, [_c_void_p] * 15 + [_c_int64] * 5 + [_c_float, _c_void_p]),
@@ -283,15 +285,22 @@ def qkv_bias_transpose(qkv, bias, stream=None):
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
 
 
-def matmul_ex(x, w, bias=None, residual=None, act: int = ACT_NONE, stream=None):
+def matmul_ex(x, w, bias=None, residual=None, act: int = ACT_NONE, stream=None, kernel: str = "auto"):
+    """kernel "auto": the measured choice between the library and the hand-written
+    MFMA kernel; "mfma": the hand-written kernel itself (fp16 / bf16, M and N
+    multiples of 128, K of 32)."""
     import torch
     M, K = x.shape
     K2, N = w.shape
     assert K == K2
     out = torch.empty((M, N), dtype=x.dtype, device=x.device)
     lib = ops()
-    fn = {torch.float16: lib.mgpuMatmulExF16, torch.bfloat16: lib.mgpuMatmulExBF16,
-          torch.float32: lib.mgpuMatmulExF32}[x.dtype]
+    if kernel == "mfma":
+        fn = {torch.float16: lib.mgpuGemmMfmaF16, torch.bfloat16: lib.mgpuGemmMfmaBF16}[x.dtype]
+    else:
+        assert kernel == "auto", kernel
+        fn = {torch.float16: lib.mgpuMatmulExF16, torch.bfloat16: lib.mgpuMatmulExBF16,
+              torch.float32: lib.mgpuMatmulExF32}[x.dtype]
     fn(_ptr(x), _ptr(w), _ptr(bias), _ptr(out), _ptr(residual), M, N, K,
        1 if bias is not None else 0, act, 1 if residual is not None else 0, _stream_handle(stream))
     _check(lib)

@@ -273,6 +273,30 @@ void mgpuMatmulExF16(void *input, void *weight, void *bias, void *output, void *
                    hasRelu, hasResidual != 0, S(stream));
   });
 }
+static void gemmMfmaChecked(mgpu::DType dt, void *input, void *weight, void *bias, void *output, void *residual,
+                            int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t act, int32_t hasResidual,
+                            hipStream_t stream) {
+  if (!input || !weight || !output) mgpu::fail("gemmMfma: null pointer");
+  if (hasBias && !bias) mgpu::fail("gemmMfma: hasBias set but bias is null");
+  if (hasResidual && !residual) mgpu::fail("gemmMfma: hasResidual set but residual is null");
+  if (act < mgpu::ACT_NONE || act > mgpu::ACT_GELU) mgpu::fail("gemmMfma: unknown activation");
+  mgpu::gemmMfma(dt, input, weight, hasBias ? bias : nullptr, hasResidual ? residual : nullptr, output, M, N, K, act,
+                 stream);
+}
+void mgpuGemmMfmaF16(void *input, void *weight, void *bias, void *output, void *residual, int64_t M, int64_t N,
+                     int64_t K, int32_t hasBias, int32_t hasRelu, int32_t hasResidual, mgpuStream_t stream) {
+  guarded([&] {
+    gemmMfmaChecked(mgpu::DType::F16, input, weight, bias, output, residual, M, N, K, hasBias, hasRelu, hasResidual,
+                    S(stream));
+  });
+}
+void mgpuGemmMfmaBF16(void *input, void *weight, void *bias, void *output, void *residual, int64_t M, int64_t N,
+                      int64_t K, int32_t hasBias, int32_t hasRelu, int32_t hasResidual, mgpuStream_t stream) {
+  guarded([&] {
+    gemmMfmaChecked(mgpu::DType::BF16, input, weight, bias, output, residual, M, N, K, hasBias, hasRelu, hasResidual,
+                    S(stream));
+  });
+}
 void mgpuMatmulExBF16(void *input, void *weight, void *bias, void *output, void *residual,
                       int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
                       int32_t hasResidual, mgpuStream_t stream) {

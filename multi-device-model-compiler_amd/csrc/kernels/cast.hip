@@ -219,7 +219,7 @@ __global__ __launch_bounds__(256) void gelu_h_vec8_kernel(u32x4 *__restrict__ da
     float v[8];
     ElemTraits<T>::unpack(data[i], v);
 #pragma unroll
-    for (int e = 0; e < 8; e++) v[e] = gelu_erf(v[e]);
+    for (int e = 0; e < 8; e++) v[e] = gelu_erfc(v[e]);
     data[i] = ElemTraits<T>::pack(v);
   }
 }
@@ -229,7 +229,11 @@ __global__ __launch_bounds__(256) void gelu_scalar_kernel(T *__restrict__ data, 
                                                           size_t n) {
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (size_t i = begin + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
-    data[i] = ElemTraits<T>::fromFloat(gelu_erf(ElemTraits<T>::toFloat(data[i])));
+  {
+    const float x = ElemTraits<T>::toFloat(data[i]);
+    // fp32 results keep the library erf; the 16-bit types take the same formula as their vector kernel
+    data[i] = ElemTraits<T>::fromFloat(sizeof(T) == 4 ? gelu_erf(x) : gelu_erfc(x));
+  }
 }
 
 } // namespace

@@ -12,13 +12,19 @@
 //    library's top candidates on scratch operands of that shape and keeps the
 //    fastest (the heuristic's first answer is not always it at M = 4096);
 //  * GELU is applied by an exact-erf kernel after a bias-only epilogue, because
-//    the library's fused GELU is the tanh approximation.
+//    the library's fused GELU is the tanh approximation;
+//  * fp16 / bf16 shapes that the hand-written MFMA kernel (gemm_mfma.hip)
+//    accepts are timed on it as well, GELU pass included on the library's
+//    side, and the faster path is kept for the shape.  MGPU_GEMM_KERNEL=library
+//    or =mfma in the environment overrides the measurement.
 #include "common.hpp"
 #include "mgpu_ops_internal.hpp"
 
 #include <hipblaslt/hipblaslt.h>
 
 #include <algorithm>
+#include <cstdlib>
+#include <cstring>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -43,7 +49,20 @@ struct Plan {
   hipblasLtMatmulDesc_t op = nullptr;
   hipblasLtMatrixLayout_t a = nullptr, b = nullptr, d = nullptr;
   hipblasLtMatmulAlgo_t algo;
+  bool handWritten = false; // serve the shape with gemm_mfma.hip when the operands allow it
 };
+
+// 0: measure, 1: always the library, 2: the hand-written kernel wherever it applies
+int forcedKernel() {
+  static const int mode = [] {
+    const char *v = std::getenv("MGPU_GEMM_KERNEL");
+    if (!v) return 0;
+    if (!std::strcmp(v, "library")) return 1;
+    if (!std::strcmp(v, "mfma")) return 2;
+    return 0;
+  }();
+  return mode;
+}
 
 using Key = std::tuple<int64_t, int64_t, int64_t, int, int, int, int>;
 std::map<Key, Plan> plans;
@@ -72,9 +91,12 @@ constexpr int kFinalists = 4;   // re-timed at length after the screening pass
 
 // Times the candidates on scratch operands of the plan's shape (its own stream,
 // its own buffers: the caller's data and stream are not touched) and returns
-// the index of the fastest; 0 when nothing could be measured.
+// the index of the fastest; 0 when nothing could be measured.  *handWritten
+// says whether the hand-written kernel beat it (with the separate GELU pass
+// counted on the library's side).
 int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *results, int count, DType dt,
-                     int64_t M, int64_t N, int64_t K, bool hasBias, bool hasResidual) {
+                     int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual,
+                     bool *handWritten) {
   const size_t eb = dt == DType::F32 ? 4 : 2;
   void *in = nullptr, *w = nullptr, *out = nullptr, *bias = nullptr;
   hipStream_t s = nullptr;
@@ -124,6 +146,35 @@ int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *resu
         best = screened[i].second;
       }
     }
+    // The hand-written kernel on the same operands (`out` doubles as the residual).
+    const void *biasArg = hasBias ? bias : nullptr, *resArg = hasResidual ? out : nullptr;
+    if (bestMs >= 0.0f && gemmMfmaSupports(dt, in, w, biasArg, resArg, out, M, N, K)) {
+      auto timeLoop = [&](auto &&launchOnce) -> float {
+        try {
+          for (int rep = 0; rep <= 20; rep++) {
+            if (rep == 1) (void)hipEventRecord(e0, s);
+            launchOnce();
+          }
+        } catch (const std::exception &) {
+          return -1.0f;
+        }
+        float ms = 0.0f;
+        if (hipEventRecord(e1, s) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+            hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
+          return -1.0f;
+        return ms / 20;
+      };
+      float libraryMs = bestMs;
+      if (act == ACT_GELU) {
+        const float geluMs = timeLoop([&] {
+          if (dt == DType::F16) geluInPlaceF16(out, (size_t)M * N, s);
+          else geluInPlaceBF16(out, (size_t)M * N, s);
+        });
+        libraryMs = geluMs >= 0.0f ? libraryMs + geluMs : -1.0f;
+      }
+      const float mfmaMs = timeLoop([&] { gemmMfma(dt, in, w, biasArg, resArg, out, M, N, K, act, s); });
+      *handWritten = libraryMs >= 0.0f && mfmaMs >= 0.0f && mfmaMs < libraryMs;
+    }
     (void)hipStreamSynchronize(s);
   }
   if (e0) (void)hipEventDestroy(e0);
@@ -135,9 +186,10 @@ int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *resu
   return best;
 }
 
-const Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, bool relu,
+const Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act,
                     bool hasResidual, hipStream_t stream) {
-  const Key key{M, N, K, (int)hasBias, (int)relu, (int)hasResidual, (int)dt};
+  const bool relu = act == ACT_RELU;
+  const Key key{M, N, K, (int)hasBias, act, (int)hasResidual, (int)dt};
   auto it = plans.find(key);
   if (it != plans.end()) return it->second;
 
@@ -182,8 +234,9 @@ const Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, boo
   p.algo = results[0].algo;
   hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
   const bool capturing = hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone;
-  if (returned > 1 && !capturing) // a capturing caller gets the heuristic's first answer
-    p.algo = results[fastestCandidate(p, results, returned, dt, M, N, K, hasBias, hasResidual)].algo;
+  if (!capturing) // a capturing caller gets the heuristic's first answer
+    p.algo = results[fastestCandidate(p, results, returned, dt, M, N, K, hasBias, act, hasResidual, &p.handWritten)].algo;
+  if (forcedKernel()) p.handWritten = forcedKernel() == 2;
   return plans.emplace(key, p).first->second;
 }
 
@@ -220,7 +273,13 @@ void matmulEx(DType dt, const void *input, const void *weight, const void *bias,
     fail("matmul: an activation cannot be combined with a residual");
 
   std::lock_guard<std::mutex> lock(planMutex);
-  const Plan &p = getPlan(dt, M, N, K, hasBias, act == ACT_RELU, hasResidual, stream);
+  const Plan &p = getPlan(dt, M, N, K, hasBias, act, hasResidual, stream);
+  if (p.handWritten && gemmMfmaSupports(dt, input, weight, hasBias ? bias : nullptr,
+                                        hasResidual ? residual : nullptr, output, M, N, K)) {
+    gemmMfma(dt, input, weight, hasBias ? bias : nullptr, hasResidual ? residual : nullptr, output, M, N, K, act,
+             stream);
+    return;
+  }
   if (hasBias)
     MGPU_CHECK_BLAS(hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias,
                                                     sizeof(bias)));

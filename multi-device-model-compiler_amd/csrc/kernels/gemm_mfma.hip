@@ -1,0 +1,307 @@
+// fp16 / bf16 GEMM with the bias, activation and residual epilogue fused, on
+// gfx950 MFMA: out[M,N] = act(in[M,K] . W[K,N] + bias[N]) (+ residual[M,N]).
+//
+// One of the two ways mgpuMatmulEx<half> (lib/Kernels/GPU/Ops.cu:134-234) is
+// served; the other is the library GEMM in gemm.cpp, and gemm.cpp times both
+// on the first use of a shape.  This kernel exists for the shapes of a
+// transformer layer at a few thousand tokens (M = 4096, N and K between 768
+// and 3072), where a GEMM is a few hundred 128x128 tiles - one to three per
+// CU - and the time goes to ramp-up, tail and the epilogue rather than to a
+// long steady state; and for the exact-erf GELU, which the library cannot fuse.
+//
+// Work decomposition.  A 256-thread block (4 wavefronts, 2 x 2) owns a
+// 128 x 128 output tile, a wavefront 64 x 64 of it as 2 x 2 accumulators of
+// 32 x 32.  The reduction runs in steps of 32: per step an 8 KiB slice of the
+// input (128 rows of 64 bytes) and an 8 KiB slice of the weight (32 rows of
+// 256 bytes) travel HBM -> LDS directly (global_load_lds, 16 bytes per lane)
+// into a ring of three stages, two steps in flight behind the one consumed;
+// three blocks share a CU (48 KiB of LDS, < 128 VGPRs).
+//
+// MFMA formulation: the transposed product out^T[n, m] = W^T[n, k] . in^T[k, m],
+//   A operand = W^T: the weight slice sits in LDS row-major as in memory
+//     ([k][n], n contiguous); ds_read_b64_tr_b16 hands lane (n = l % 32) the
+//     four k of its column, two reads per operand;
+//   B operand = in^T: lane (m = l % 32) reads 16 contiguous bytes of its row.
+// so that an accumulator register group holds four consecutive n of one row m:
+// bias, activation and residual are applied on 8-byte pieces of output rows,
+// and the tile is then transposed through LDS so that every store instruction
+// writes whole 128-byte runs of output rows.  Both slices are stored unpadded
+// (the direct loads fill 1 KiB of consecutive LDS per instruction) with an XOR
+// swizzle on the 16-byte chunk index that keeps both operand reads free of
+// bank conflicts.
+//
+// Shapes: M and N multiples of 128, K a multiple of 32, 16-byte aligned
+// operands.  Everything else goes to the library.
+#include "common.hpp"
+#include "mfma.hpp"
+#include "mgpu_ops_internal.hpp"
+#include "types.hpp"
+
+namespace mgpu {
+
+namespace {
+
+constexpr int kBM = 128, kBN = 128, kBK = 32;
+constexpr int kRing = 3;           // LDS ring depth
+constexpr int kSlice = 8192;       // one input or weight slice
+constexpr int kARow = kBK * 2;     // bytes per row of the input slice: 64
+constexpr int kWRow = kBN * 2;     // bytes per row of the weight slice: 256
+constexpr int kOutStride = 64 + 4; // staging row stride of a wavefront's 64 x 64 tile, in elements
+
+// Chunk swizzles: the 16-byte chunk c of a row is kept at chunk c ^ swz(row).
+__host__ __device__ constexpr int aSwz(int row) { return (row >> 2) & 3; }        // 4 chunks per row
+__host__ __device__ constexpr int wSwz(int row) { return (row & 3) << 2; }        // 16 chunks per row
+
+template <typename T, int ACT>
+__global__ __launch_bounds__(256, 3) void gemm_mfma_kernel(const uint16_t *__restrict__ in,
+                                                           const uint16_t *__restrict__ weight,
+                                                           const uint16_t *__restrict__ bias,
+                                                           const uint16_t *residual, uint16_t *out, int N, int K, int tilesN) {
+  using M = Mma<T>;
+  using v8 = typename M::v8;
+  using v4 = typename M::v4;
+
+  // Ring of kRing stages, each an input slice followed by a weight slice;
+  // reused as the output staging area at the end.
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[kRing * 2 * kSlice];
+  static_assert(4 * 64 * kOutStride * 2 <= kRing * 2 * kSlice, "output staging must fit in the ring");
+
+  // Tile order: the tiles of one row of tiles (same input rows) are
+  // consecutive, and a contiguous run of tiles goes to each of the 8 XCDs
+  // (consecutive block ids are dealt round-robin to the XCDs).
+  const int nblk = gridDim.x;
+  const int bid = blockIdx.x;
+  const int wid = (nblk % 8 == 0) ? (bid % 8) * (nblk / 8) + bid / 8 : bid;
+  const int m0 = (wid / tilesN) * kBM;
+  const int n0 = (wid % tilesN) * kBN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int l32 = lane % 32;
+  const int hl = lane / 32;
+  const int wm = wave >> 1, wn = wave & 1; // the wavefront's 64 x 64 quadrant
+
+  // ---- slice movers: HBM -> LDS, 16 bytes per lane ----------------------------
+  // One wavefront instruction fills 1 KiB: 16 rows of the input slice or 4 rows
+  // of the weight slice; wavefront w moves 2 KiB of both.
+  const char *abase = reinterpret_cast<const char *>(in) + (size_t)m0 * K * 2;
+  const char *wbase = reinterpret_cast<const char *>(weight) + (size_t)n0 * 2;
+  uint32_t aoff[2], woff[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int arow = 16 * (2 * wave + i) + lane / 4;
+    aoff[i] = (uint32_t)arow * (uint32_t)K * 2u + (uint32_t)(((lane % 4) ^ aSwz(arow)) * 16);
+    const int wrow = 4 * (2 * wave + i) + lane / 16;
+    woff[i] = (uint32_t)wrow * (uint32_t)N * 2u + (uint32_t)(((lane % 16) ^ wSwz(wrow)) * 16);
+  }
+  // Inline assembly keeps these loads out of the compiler's wait-count
+  // bookkeeping, which would otherwise wait for every load in flight before
+  // any later LDS read; completion is tracked by hand (4 loads per stage and
+  // wavefront).
+  const uint32_t ldsBase = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) unsigned char *)smem);
+  auto dma16 = [&](uint32_t voffset, const char *sbase, uint32_t ldsAddr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voffset), "s"(sbase), "s"(ldsAddr)
+                 : "memory");
+  };
+  auto issueStage = [&](int kt) {
+    const uint32_t adst = ldsBase + (uint32_t)((kt % kRing) * (2 * kSlice) + (2 * wave) * 1024);
+    const uint32_t wdst = adst + kSlice;
+    const char *ag = abase + (size_t)kt * kARow;
+    const char *wg = wbase + (size_t)kt * kBK * N * 2;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      dma16(aoff[i], ag, adst + i * 1024);
+      dma16(woff[i], wg, wdst + i * 1024);
+    }
+  };
+
+  const int nk = K / kBK;
+#pragma unroll
+  for (int t = 0; t < kRing - 1; t++)
+    if (t < nk) issueStage(t);
+
+  // ---- operand addresses inside a stage ---------------------------------------
+  // in^T: lane (row wm*64 + 32mb + l32, k chunk 2c + hl) reads 16 bytes.
+  uint32_t afrag[2][2];
+#pragma unroll
+  for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+      const int row = wm * 64 + 32 * mb + l32;
+      afrag[mb][c] = (uint32_t)(row * kARow + (((2 * c + hl) ^ aSwz(row)) * 16));
+    }
+  // W^T: as a source of the transposing read, lane L of a 16-lane group g points
+  // at k row 8*hl + L/4 (+ 16c, + 4 for the upper k-slots) and the four columns
+  // n = 32nb + 16*(g%2) + 4*(L%4) .. +3.
+  uint32_t wfrag[2];
+  {
+    const int g = lane / 16, L = lane % 16, r = L % 4, j = L / 4;
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+      const int chunk = (4 * (2 * wn + nb) + 2 * (g % 2) + r / 2) ^ wSwz(j);
+      wfrag[nb] = (uint32_t)(kSlice + (8 * hl + j) * kWRow + chunk * 16 + 8 * (r % 2));
+    }
+  }
+
+  f32x16 acc[2][2]; // [nb][mb]: rows n, columns m
+#pragma unroll
+  for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+    for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) acc[nb][mb][i] = 0.0f;
+
+  for (int kt = 0; kt < nk; kt++) {
+    // The loads of stage kt (and of nothing later) must have landed; the barrier
+    // makes every wavefront's share visible and says that everybody is done
+    // with stage kt-1, which the next load overwrites.
+    if (kt + 1 < nk) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (kt + kRing - 1 < nk) issueStage(kt + kRing - 1);
+
+    const uint32_t stageBase = ldsBase + (uint32_t)((kt % kRing) * (2 * kSlice));
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+      v8 b[2], a[2];
+#pragma unroll
+      for (int mb = 0; mb < 2; mb++)
+        b[mb] = *reinterpret_cast<const v8 __attribute__((address_space(3))) *>(
+            (const lds_u8 *)(uintptr_t)(stageBase + afrag[mb][c]));
+#pragma unroll
+      for (int nb = 0; nb < 2; nb++) {
+        const lds_u8 *p = (const lds_u8 *)(uintptr_t)(stageBase + wfrag[nb]) + 16 * c * kWRow;
+        const v4 lo = M::readTr(p);             // k-slots 0..3
+        const v4 hi = M::readTr(p + 4 * kWRow); // k-slots 4..7
+        a[nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+#pragma unroll
+      for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++) acc[nb][mb] = M::run(a[nb], b[mb], acc[nb][mb]);
+    }
+  }
+
+  // ---- epilogue: bias, activation, residual; transpose through LDS; store ------
+  __syncthreads(); // every wavefront is done reading the slices
+  uint16_t *stage = reinterpret_cast<uint16_t *>(smem) + wave * (64 * kOutStride);
+  const int mw = m0 + wm * 64, nw = n0 + wn * 64; // origin of the wavefront's quadrant
+  // All bias pieces of the quadrant first, then per 32-column block all of its
+  // residual pieces, so that the loads of a batch are in flight together.
+  v4 braw[2][4];
+#pragma unroll
+  for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) braw[nb][g][i] = M::narrow(0.0f);
+  if (bias) {
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) braw[nb][g] = *reinterpret_cast<const v4 *>(bias + nw + 32 * nb + 8 * g + 4 * hl);
+  }
+#pragma unroll
+  for (int nb = 0; nb < 2; nb++) {
+    v4 rraw[4][2];
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+#pragma unroll
+      for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) rraw[g][mb][i] = M::narrow(0.0f);
+    if (residual) {
+#pragma unroll
+      for (int g = 0; g < 4; g++)
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++)
+          rraw[g][mb] = *reinterpret_cast<const v4 *>(residual + (size_t)(mw + 32 * mb + l32) * N + nw + 32 * nb +
+                                                      8 * g + 4 * hl);
+    }
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      const int nloc = 32 * nb + 8 * g + 4 * hl; // four consecutive columns of the quadrant
+#pragma unroll
+      for (int mb = 0; mb < 2; mb++) {
+        const int mloc = 32 * mb + l32;
+        float x[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = acc[nb][mb][4 * g + i] + M::widen(braw[nb][g][i]);
+        if (ACT == ACT_RELU) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) x[i] = x[i] > 0.0f ? x[i] : 0.0f;
+        } else if (ACT == ACT_GELU) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) x[i] = gelu_erfc(x[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] += M::widen(rraw[g][mb][i]);
+        v4 o;
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = M::narrow(x[i]);
+        *reinterpret_cast<v4 *>(&stage[mloc * kOutStride + nloc]) = o;
+      }
+    }
+  }
+  // Each wavefront reads back only what it wrote: no block barrier needed, the
+  // LDS accesses of one wavefront are ordered.
+#pragma unroll
+  for (int it = 0; it < 8; it++) {
+    const int chunk = it * 64 + lane; // 16-byte chunk of the quadrant: 64 rows x 8
+    const int r = chunk / 8, cidx = chunk % 8;
+    // 8-byte LDS reads: the staging stride is 8-byte but not 16-byte aligned
+    const u32x2 lo = *reinterpret_cast<const u32x2 *>(&stage[r * kOutStride + cidx * 8]);
+    const u32x2 hi = *reinterpret_cast<const u32x2 *>(&stage[r * kOutStride + cidx * 8 + 4]);
+    const u32x4 val = {lo[0], lo[1], hi[0], hi[1]};
+    *reinterpret_cast<u32x4 *>(out + (size_t)(mw + r) * N + nw + cidx * 8) = val;
+  }
+}
+
+template <typename T>
+void launch(const void *in, const void *weight, const void *bias, const void *residual, void *out, int64_t M,
+            int64_t N, int64_t K, int act, hipStream_t stream) {
+  const int tilesN = (int)(N / kBN);
+  const unsigned blocks = (unsigned)((M / kBM) * tilesN);
+  const auto *a = static_cast<const uint16_t *>(in);
+  const auto *w = static_cast<const uint16_t *>(weight);
+  const auto *b = static_cast<const uint16_t *>(bias);
+  const auto *r = static_cast<const uint16_t *>(residual);
+  auto *o = static_cast<uint16_t *>(out);
+  if (act == ACT_GELU)
+    gemm_mfma_kernel<T, ACT_GELU><<<dim3(blocks), dim3(256), 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+  else if (act == ACT_RELU)
+    gemm_mfma_kernel<T, ACT_RELU><<<dim3(blocks), dim3(256), 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+  else
+    gemm_mfma_kernel<T, ACT_NONE><<<dim3(blocks), dim3(256), 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+  MGPU_CHECK_LAUNCH("gemm_mfma_kernel");
+}
+
+} // namespace
+
+bool gemmMfmaSupports(DType dt, const void *in, const void *weight, const void *bias, const void *residual,
+                      const void *out, int64_t M, int64_t N, int64_t K) {
+  if (dt != DType::F16 && dt != DType::BF16) return false;
+  if (M <= 0 || N <= 0 || K <= 0 || M % kBM || N % kBN || K % kBK) return false;
+  // 32-bit lane offsets inside a slice, 31-bit tile counts
+  if (K > (1 << 20) || N > (1 << 20) || (M / kBM) * (N / kBN) > 0x7fffffffLL) return false;
+  if (!aligned16(in) || !aligned16(weight) || !aligned16(out)) return false;
+  if (bias && (reinterpret_cast<uintptr_t>(bias) & 7u)) return false;
+  if (residual && !aligned16(residual)) return false;
+  return true;
+}
+
+void gemmMfma(DType dt, const void *in, const void *weight, const void *bias, const void *residual, void *out,
+              int64_t M, int64_t N, int64_t K, int act, hipStream_t stream) {
+  if (!gemmMfmaSupports(dt, in, weight, bias, residual, out, M, N, K))
+    fail("gemmMfma: shape, type or alignment not supported by the hand-written kernel");
+  if (act != ACT_NONE && residual) fail("gemmMfma: an activation cannot be combined with a residual");
+  if (dt == DType::F16)
+    launch<_Float16>(in, weight, bias, residual, out, M, N, K, act, stream);
+  else
+    launch<bf16_t>(in, weight, bias, residual, out, M, N, K, act, stream);
+}
+
+} // namespace mgpu

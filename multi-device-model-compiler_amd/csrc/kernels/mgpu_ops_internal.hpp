@@ -41,6 +41,13 @@ void matmulEx(DType dt, const void *input, const void *weight, const void *bias,
               const void *residual, int64_t M, int64_t N, int64_t K, bool hasBias, int act,
               bool hasResidual, hipStream_t stream);
 
+// Hand-written MFMA GEMM (gemm_mfma.hip): fp16 / bf16, M and N multiples of 128,
+// K a multiple of 32, 16-byte aligned operands; bias and residual may be null.
+bool gemmMfmaSupports(DType dt, const void *in, const void *weight, const void *bias, const void *residual,
+                      const void *out, int64_t M, int64_t N, int64_t K);
+void gemmMfma(DType dt, const void *in, const void *weight, const void *bias, const void *residual, void *out,
+              int64_t M, int64_t N, int64_t K, int act, hipStream_t stream);
+
 void conv2d(const float *input, const float *weight, const float *bias, float *output, const float *postAdd,
             int64_t N, int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t OH,
             int64_t OW, int64_t PHL, int64_t PWL, int64_t PHR, int64_t PWR, int64_t SH, int64_t SW, int64_t DH,

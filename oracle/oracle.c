@@ -350,7 +350,9 @@ ORACLE_API void oracle_fmha(const void *qkv, const int32_t *seqlens, float *out,
 /* GEMM with epilogue, casts, QKV transpose                            */
 /* ------------------------------------------------------------------ */
 
-static inline double gelu_erf(double x) { return 0.5 * x * (1.0 + erf(x * 0.70710678118654752440)); }
+/* x * Phi(x); 1 + erf(z) written as erfc(-z), which keeps its relative
+ * accuracy on the negative tail instead of cancelling. */
+static inline double gelu_erf(double x) { return 0.5 * x * erfc(-x * 0.70710678118654752440); }
 
 /* out[M,N] = act(in[M,K] . W[K,N] + bias[N]) + residual[M,N], all row major:
  * the contract of lib/Kernels/GPU/Ops.cu:134-234 (row-major via the swapped

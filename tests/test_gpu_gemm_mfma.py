@@ -1,0 +1,129 @@
+"""The hand-written MFMA GEMM (mgpuGemmMfmaF16 / BF16) against the oracle's GEMM,
+through the C ABI: every epilogue, both types, shapes from one tile and one
+reduction step up to the BERT-base layer's, and the shapes it must refuse."""
+import numpy as np
+import pytest
+
+from conftest import to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def bf16_bits(t):
+    import torch
+    return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def spacing_tol(ref, mant_bits, floor):
+    """One spacing of the 16-bit result type at the reference's magnitude, plus a floor."""
+    e = np.floor(np.log2(np.maximum(np.abs(ref), 2.0 ** -14)))
+    return 2.0 ** (e - mant_bits) + floor
+
+
+SHAPES = [(128, 32, 128), (128, 64, 256), (256, 96, 384), (384, 160, 128), (256, 1024, 128), (512, 768, 768),
+          (1024, 768, 3072), (4096, 768, 2304)]
+
+
+def epilogues(pkg, oracle, tb, b, tr, r):
+    return [(dict(), dict()), (dict(bias=tb), dict(bias=b)), (dict(residual=tr), dict(residual=r)),
+            (dict(bias=tb, act=pkg.ACT_RELU), dict(bias=b, act=oracle.ACT_RELU)),
+            (dict(act=pkg.ACT_GELU), dict(act=oracle.ACT_GELU)),
+            (dict(bias=tb, act=pkg.ACT_GELU), dict(bias=b, act=oracle.ACT_GELU)),
+            (dict(bias=tb, residual=tr), dict(bias=b, residual=r))]
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+def test_gemm_mfma_f16(pkg, gpu, oracle, rng, M, K, N):
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    b = rng.standard_normal(N).astype(np.float16)
+    r = rng.standard_normal((M, N)).astype(np.float16)
+    tx, tw, tb, tr = [to_dev(t, gpu) for t in (x, w, b, r)]
+    for kw, okw in epilogues(pkg, oracle, tb, b, tr, r):
+        got = pkg.matmul_ex(tx, tw, kernel="mfma", **kw).cpu().numpy().astype(np.float32)
+        ref = oracle.gemm(x, w, **okw)
+        # fp32 accumulation, epilogue in fp32, one rounding: one fp16 spacing of the result
+        err = np.abs(got - ref)
+        assert np.all(err <= spacing_tol(ref, 10, 1e-3)), (sorted(kw), err.max())
+
+
+@pytest.mark.parametrize("M,K,N", [(128, 32, 128), (256, 96, 384), (512, 768, 768)])
+def test_gemm_mfma_bf16(pkg, gpu, oracle, rng, M, K, N):
+    import torch
+    mk = lambda a: torch.from_numpy(a.astype(np.float32)).to(gpu).to(torch.bfloat16)
+    tx, tw = mk(rng.standard_normal((M, K))), mk(rng.standard_normal((K, N)) / np.sqrt(K))
+    tb, tr = mk(rng.standard_normal(N)), mk(rng.standard_normal((M, N)))
+    x, w, b, r = [bf16_bits(t) for t in (tx, tw, tb, tr)]
+    for kw, okw in epilogues(pkg, oracle, tb, b, tr, r):
+        got = pkg.matmul_ex(tx, tw, kernel="mfma", **kw).float().cpu().numpy()
+        ref = oracle.gemm(x, w, bf16=True, **okw)
+        err = np.abs(got - ref)
+        assert np.all(err <= spacing_tol(ref, 7, 4e-3)), (sorted(kw), err.max())
+
+
+def test_gemm_mfma_matches_library_path(pkg, gpu, rng):
+    """The measured choice behind mgpuMatmulExF16 may be either kernel: without an
+    activation both round the same fp32 sums once, so they agree to the last bit
+    wherever the two summation orders round alike, and to one spacing elsewhere."""
+    M, K, N = 512, 768, 768
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    b = rng.standard_normal(N).astype(np.float16)
+    tx, tw, tb = [to_dev(t, gpu) for t in (x, w, b)]
+    a = pkg.matmul_ex(tx, tw, bias=tb).cpu().numpy().astype(np.float32)
+    m = pkg.matmul_ex(tx, tw, bias=tb, kernel="mfma").cpu().numpy().astype(np.float32)
+    assert np.all(np.abs(a - m) <= spacing_tol(m, 10, 0.0))
+    assert np.mean(a == m) > 0.99
+
+
+def test_gemm_mfma_in_place_residual(pkg, gpu, oracle, rng):
+    """The residual may be the output buffer itself (C == D), as the library path allows."""
+    import torch
+    M, K, N = 256, 64, 256
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    r = rng.standard_normal((M, N)).astype(np.float16)
+    tx, tw, out = to_dev(x, gpu), to_dev(w, gpu), to_dev(r, gpu)
+    lib = pkg.ops()
+    lib.mgpuGemmMfmaF16(tx.data_ptr(), tw.data_ptr(), None, out.data_ptr(), out.data_ptr(), M, N, K, 0, 0, 1,
+                        torch.cuda.current_stream().cuda_stream)
+    assert lib.mgpuOpsTakeLastError() is None
+    torch.cuda.synchronize()
+    ref = oracle.gemm(x, w, residual=r)
+    assert np.all(np.abs(out.cpu().numpy().astype(np.float32) - ref) <= spacing_tol(ref, 10, 1e-3))
+
+
+@pytest.mark.parametrize("M,K,N", [(100, 64, 128), (128, 48, 128), (128, 64, 72), (128, 0, 128)])
+def test_gemm_mfma_refuses_other_shapes(pkg, gpu, M, K, N):
+    import torch
+    x = torch.zeros((M, max(K, 1)), dtype=torch.float16, device=gpu)[:, :K].contiguous()
+    w = torch.zeros((max(K, 1), N), dtype=torch.float16, device=gpu)[:K].contiguous()
+    with pytest.raises(pkg.MgpuError):
+        pkg.matmul_ex(x, w, kernel="mfma")
+
+
+def test_gemm_mfma_refuses_fp32_and_activation_with_residual(pkg, gpu):
+    import torch
+    x = torch.zeros((128, 32), dtype=torch.float16, device=gpu)
+    w = torch.zeros((32, 128), dtype=torch.float16, device=gpu)
+    r = torch.zeros((128, 128), dtype=torch.float16, device=gpu)
+    with pytest.raises(pkg.MgpuError):
+        pkg.matmul_ex(x, w, residual=r, act=pkg.ACT_RELU, kernel="mfma")
+    with pytest.raises(KeyError):
+        pkg.matmul_ex(x.float(), w.float(), kernel="mfma")
+
+
+def test_gelu_erfc_form_tail(pkg, gpu, oracle):
+    """x * Phi(x) on the negative tail, where 1 + erf cancels: a bias-only GEMM of
+    zeros puts chosen values through the fused GELU."""
+    import torch
+    M, K, N = 128, 32, 128
+    vals = np.linspace(-9.0, 9.0, N).astype(np.float16)
+    x = torch.zeros((M, K), dtype=torch.float16, device=gpu)
+    w = torch.zeros((K, N), dtype=torch.float16, device=gpu)
+    got = pkg.matmul_ex(x, w, bias=to_dev(vals, gpu), act=pkg.ACT_GELU, kernel="mfma").cpu().numpy()
+    ref = oracle.gemm(np.zeros((M, K), np.float16), np.zeros((K, N), np.float16), bias=vals, act=oracle.ACT_GELU)
+    want = ref.astype(np.float16)
+    # at most one unit in the last place of the fp16 result, subnormals included
+    ulps = np.abs(got.view(np.int16).astype(np.int32) - want.view(np.int16).astype(np.int32))
+    assert ulps.max() <= 1, ulps.max()
