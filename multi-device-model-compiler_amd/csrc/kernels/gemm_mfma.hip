@@ -66,14 +66,23 @@ __global__ __launch_bounds__(256, 3) void gemm_mfma_kernel(const uint16_t *__res
   __shared__ __attribute__((aligned(1024))) unsigned char smem[kRing * 2 * kSlice];
   static_assert(4 * 64 * kOutStride * 2 <= kRing * 2 * kSlice, "output staging must fit in the ring");
 
-  // Tile order: the tiles of one row of tiles (same input rows) are
-  // consecutive, and a contiguous run of tiles goes to each of the 8 XCDs
-  // (consecutive block ids are dealt round-robin to the XCDs).
+  // Tile order.  A contiguous run of work items goes to each of the 8 XCDs
+  // (consecutive block ids are dealt round-robin to the XCDs), and consecutive
+  // work items walk down kGroup rows of tiles before stepping one column, so
+  // that the ~96 blocks resident on an XCD form a compact patch of tiles: the
+  // slices they load per step are then few (8 input + 12 weight slices instead
+  // of 2 + 64 for a row-major sweep of a wide matrix) and hit in that XCD's L2.
+  constexpr int kGroup = 8;
   const int nblk = gridDim.x;
   const int bid = blockIdx.x;
   const int wid = (nblk % 8 == 0) ? (bid % 8) * (nblk / 8) + bid / 8 : bid;
-  const int m0 = (wid / tilesN) * kBM;
-  const int n0 = (wid % tilesN) * kBN;
+  const int tilesM = nblk / tilesN;
+  const int perGroup = kGroup * tilesN;
+  const int firstM = (wid / perGroup) * kGroup;
+  const int groupRows = tilesM - firstM < kGroup ? tilesM - firstM : kGroup;
+  const int inGroup = wid % perGroup;
+  const int m0 = (firstM + inGroup % groupRows) * kBM;
+  const int n0 = (inGroup / groupRows) * kBN;
 
   const int tid = threadIdx.x;
   const int lane = tid % 64;
