@@ -152,7 +152,7 @@ void mgpuMatmulExBF16(void *input, void *weight, void *bias, void *output, void 
 
 /* The hand-written MFMA kernel that serves mgpuMatmulExF16 / BF16 where it is
  * the faster path, callable by itself (no counterpart in the reference):
- * same arguments; M and N multiples of 128, K a multiple of 32, operands
+ * same arguments; M a multiple of 128, N of 128 or 96, K of 32, operands
  * 16-byte aligned, anything else is an error. */
 void mgpuGemmMfmaF16(void *input, void *weight, void *bias, void *output, void *residual,
                      int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,

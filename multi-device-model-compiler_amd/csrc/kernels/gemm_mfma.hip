@@ -9,13 +9,19 @@
 // CU - and the time goes to ramp-up, tail and the epilogue rather than to a
 // long steady state; and for the exact-erf GELU, which the library cannot fuse.
 //
-// Work decomposition.  A 256-thread block (4 wavefronts, 2 x 2) owns a
-// 128 x 128 output tile, a wavefront 64 x 64 of it as 2 x 2 accumulators of
-// 32 x 32.  The reduction runs in steps of 32: per step an 8 KiB slice of the
-// input (128 rows of 64 bytes) and an 8 KiB slice of the weight (32 rows of
-// 256 bytes) travel HBM -> LDS directly (global_load_lds, 16 bytes per lane)
-// into a ring of three stages, two steps in flight behind the one consumed;
-// three blocks share a CU (48 KiB of LDS, < 128 VGPRs).
+// Work decomposition.  A 256-thread block (4 wavefronts) owns a 128 x 128 output
+// tile (wavefronts 2 x 2, each 64 x 64 as 2 x 2 accumulators of 32 x 32) or a
+// 128 x 96 one (wavefronts 4 x 1, each 32 x 96 as 3 accumulators); the launcher
+// takes the width that loads the busiest CU least (768 columns are 6 tiles of
+// 128 - 192 tiles at M = 4096, a quarter of the CUs idle - or 8 of 96 - 256
+// tiles, one per CU).  The reduction runs in steps of 32: per step an 8 KiB
+// slice of the input (128 rows of 64 bytes) and a slice of the weight (32 rows
+// at a 256-byte pitch) travel HBM -> LDS directly (global_load_lds, 16 bytes per
+// lane) into a ring of three stages, two steps in flight behind the one
+// consumed; three blocks share a CU (48 KiB of LDS, < 128 VGPRs).  When there
+// is at most one tile per CU the step is 64 instead (96 KiB of LDS): a lone
+// block cannot hide the barrier and the LDS latency of a step behind other
+// blocks, so it takes half as many, longer steps.
 //
 // MFMA formulation: the transposed product out^T[n, m] = W^T[n, k] . in^T[k, m],
 //   A operand = W^T: the weight slice sits in LDS row-major as in memory
@@ -30,7 +36,7 @@
 // swizzle on the 16-byte chunk index that keeps both operand reads free of
 // bank conflicts.
 //
-// Shapes: M and N multiples of 128, K a multiple of 32, 16-byte aligned
+// Shapes: M a multiple of 128, N of 128 or 96, K of 32, 16-byte aligned
 // operands.  Everything else goes to the library.
 #include "common.hpp"
 #include "mfma.hpp"
@@ -41,30 +47,42 @@ namespace mgpu {
 
 namespace {
 
-constexpr int kBM = 128, kBN = 128, kBK = 32;
-constexpr int kRing = 3;           // LDS ring depth
-constexpr int kSlice = 8192;       // one input or weight slice
-constexpr int kARow = kBK * 2;     // bytes per row of the input slice: 64
-constexpr int kWRow = kBN * 2;     // bytes per row of the weight slice: 256
-constexpr int kOutStride = 64 + 4; // staging row stride of a wavefront's 64 x 64 tile, in elements
+constexpr int kBM = 128;       // rows of an output tile
+constexpr int kRing = 3;       // LDS ring depth
+constexpr int kWRow = 256;     // LDS pitch of a weight-slice row, bytes (128 columns, of which NB * 32 are loaded)
 
 // Chunk swizzles: the 16-byte chunk c of a row is kept at chunk c ^ swz(row).
-__host__ __device__ constexpr int aSwz(int row) { return (row >> 2) & 3; }        // 4 chunks per row
-__host__ __device__ constexpr int wSwz(int row) { return (row & 3) << 2; }        // 16 chunks per row
+template <int BK> __host__ __device__ constexpr int aSwz(int row) {
+  return BK == 32 ? (row >> 2) & 3 : (row >> 1) & 7; // 4 or 8 chunks per row
+}
+__host__ __device__ constexpr int wSwz(int row) { return (row & 3) << 2; } // 16 chunks per row
 
-template <typename T, int ACT>
-__global__ __launch_bounds__(256, 3) void gemm_mfma_kernel(const uint16_t *__restrict__ in,
-                                                           const uint16_t *__restrict__ weight,
-                                                           const uint16_t *__restrict__ bias,
-                                                           const uint16_t *residual, uint16_t *out, int N, int K, int tilesN) {
+// T: element type; ACT: epilogue activation; BK: reduction step (32 or 64);
+// NB: tile width in 32-column blocks (4 or 3).
+template <typename T, int ACT, int BK, int NB>
+__global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const uint16_t *__restrict__ in,
+                                                                        const uint16_t *__restrict__ weight,
+                                                                        const uint16_t *__restrict__ bias,
+                                                                        const uint16_t *residual, uint16_t *out, int N,
+                                                                        int K, int tilesN) {
   using M = Mma<T>;
   using v8 = typename M::v8;
   using v4 = typename M::v4;
+  static_assert((BK == 32 || BK == 64) && (NB == 4 || NB == 3), "tile geometry");
+  constexpr int kBN = 32 * NB;
+  constexpr int kSlice = 256 * BK;                   // bytes of an input slice, and of a weight slice at full pitch
+  constexpr int kARow = BK * 2;                      // bytes per row of the input slice: 64 / 128
+  constexpr int NC = BK / 16;                        // MFMA k-steps per reduction step: 2 / 4
+  constexpr int NL = BK / 16;                        // load instructions per wavefront and slice: 2 / 4
+  constexpr int CPR = BK / 8, RPI = 64 / CPR;        // input slice: chunks per row, rows per load instruction
+  constexpr int WN = NB == 4 ? 2 : 1, WM = 4 / WN;   // wavefront grid over the tile: 2 x 2 or 4 x 1
+  constexpr int MB = 4 / WM, NBW = NB / WN;          // 32 x 32 accumulators per wavefront: MB x NBW = 2 x 2 or 1 x 3
+  constexpr int kOutStride = 32 * NBW + 4;           // staging row stride of a wavefront's part, in elements
 
   // Ring of kRing stages, each an input slice followed by a weight slice;
   // reused as the output staging area at the end.
   __shared__ __attribute__((aligned(1024))) unsigned char smem[kRing * 2 * kSlice];
-  static_assert(4 * 64 * kOutStride * 2 <= kRing * 2 * kSlice, "output staging must fit in the ring");
+  static_assert(4 * 32 * MB * kOutStride * 2 <= kRing * 2 * kSlice, "output staging must fit in the ring");
 
   // Tile order.  A contiguous run of work items goes to each of the 8 XCDs
   // (consecutive block ids are dealt round-robin to the XCDs), and consecutive
@@ -89,25 +107,31 @@ __global__ __launch_bounds__(256, 3) void gemm_mfma_kernel(const uint16_t *__res
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int l32 = lane % 32;
   const int hl = lane / 32;
-  const int wm = wave >> 1, wn = wave & 1; // the wavefront's 64 x 64 quadrant
+  const int wm = wave / WN, wn = wave % WN; // the wavefront's part of the tile
 
   // ---- slice movers: HBM -> LDS, 16 bytes per lane ----------------------------
-  // One wavefront instruction fills 1 KiB: 16 rows of the input slice or 4 rows
-  // of the weight slice; wavefront w moves 2 KiB of both.
+  // One wavefront instruction fills 1 KiB: RPI rows of the input slice or 4 rows
+  // of the weight slice; every wavefront moves a quarter of both.  In a 96-column
+  // tile the lanes that would fetch the chunks beyond column 95 fetch a chunk of
+  // the tile again instead: it lands in the unread tail of the 256-byte pitch.
+  // (Masking those lanes off would put the load under divergent control flow,
+  // where its scalar operands are no longer scalar to the compiler.)
   const char *abase = reinterpret_cast<const char *>(in) + (size_t)m0 * K * 2;
   const char *wbase = reinterpret_cast<const char *>(weight) + (size_t)n0 * 2;
-  uint32_t aoff[2], woff[2];
+  uint32_t aoff[NL], woff[NL];
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
-    const int arow = 16 * (2 * wave + i) + lane / 4;
-    aoff[i] = (uint32_t)arow * (uint32_t)K * 2u + (uint32_t)(((lane % 4) ^ aSwz(arow)) * 16);
-    const int wrow = 4 * (2 * wave + i) + lane / 16;
-    woff[i] = (uint32_t)wrow * (uint32_t)N * 2u + (uint32_t)(((lane % 16) ^ wSwz(wrow)) * 16);
+  for (int i = 0; i < NL; i++) {
+    const int arow = RPI * (NL * wave + i) + lane / CPR;
+    aoff[i] = (uint32_t)arow * (uint32_t)K * 2u + (uint32_t)(((lane % CPR) ^ aSwz<BK>(arow)) * 16);
+    const int wrow = 4 * (NL * wave + i) + lane / 16;
+    int wchunk = (lane % 16) ^ wSwz(wrow);
+    if (wchunk >= 4 * NB) wchunk -= 4;
+    woff[i] = (uint32_t)wrow * (uint32_t)N * 2u + (uint32_t)(wchunk * 16);
   }
   // Inline assembly keeps these loads out of the compiler's wait-count
   // bookkeeping, which would otherwise wait for every load in flight before
-  // any later LDS read; completion is tracked by hand (4 loads per stage and
-  // wavefront).
+  // any later LDS read; completion is tracked by hand (2 * NL loads per stage
+  // and wavefront).
   const uint32_t ldsBase = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) unsigned char *)smem);
   auto dma16 = [&](uint32_t voffset, const char *sbase, uint32_t ldsAddr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
@@ -116,50 +140,50 @@ __global__ __launch_bounds__(256, 3) void gemm_mfma_kernel(const uint16_t *__res
                  : "memory");
   };
   auto issueStage = [&](int kt) {
-    const uint32_t adst = ldsBase + (uint32_t)((kt % kRing) * (2 * kSlice) + (2 * wave) * 1024);
+    const uint32_t adst = ldsBase + (uint32_t)((kt % kRing) * (2 * kSlice) + (NL * wave) * 1024);
     const uint32_t wdst = adst + kSlice;
     const char *ag = abase + (size_t)kt * kARow;
-    const char *wg = wbase + (size_t)kt * kBK * N * 2;
+    const char *wg = wbase + (size_t)kt * BK * N * 2;
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
+    for (int i = 0; i < NL; i++) {
       dma16(aoff[i], ag, adst + i * 1024);
       dma16(woff[i], wg, wdst + i * 1024);
     }
   };
 
-  const int nk = K / kBK;
+  const int nk = K / BK;
 #pragma unroll
   for (int t = 0; t < kRing - 1; t++)
     if (t < nk) issueStage(t);
 
   // ---- operand addresses inside a stage ---------------------------------------
-  // in^T: lane (row wm*64 + 32mb + l32, k chunk 2c + hl) reads 16 bytes.
-  uint32_t afrag[2][2];
+  // in^T: lane (row 32*MB*wm + 32mb + l32, k chunk 2c + hl) reads 16 bytes.
+  uint32_t afrag[MB][NC];
 #pragma unroll
-  for (int mb = 0; mb < 2; mb++)
+  for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-    for (int c = 0; c < 2; c++) {
-      const int row = wm * 64 + 32 * mb + l32;
-      afrag[mb][c] = (uint32_t)(row * kARow + (((2 * c + hl) ^ aSwz(row)) * 16));
+    for (int c = 0; c < NC; c++) {
+      const int row = wm * (32 * MB) + 32 * mb + l32;
+      afrag[mb][c] = (uint32_t)(row * kARow + (((2 * c + hl) ^ aSwz<BK>(row)) * 16));
     }
   // W^T: as a source of the transposing read, lane L of a 16-lane group g points
   // at k row 8*hl + L/4 (+ 16c, + 4 for the upper k-slots) and the four columns
   // n = 32nb + 16*(g%2) + 4*(L%4) .. +3.
-  uint32_t wfrag[2];
+  uint32_t wfrag[NBW];
   {
     const int g = lane / 16, L = lane % 16, r = L % 4, j = L / 4;
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
-      const int chunk = (4 * (2 * wn + nb) + 2 * (g % 2) + r / 2) ^ wSwz(j);
+    for (int nb = 0; nb < NBW; nb++) {
+      const int chunk = (4 * (NBW * wn + nb) + 2 * (g % 2) + r / 2) ^ wSwz(j);
       wfrag[nb] = (uint32_t)(kSlice + (8 * hl + j) * kWRow + chunk * 16 + 8 * (r % 2));
     }
   }
 
-  f32x16 acc[2][2]; // [nb][mb]: rows n, columns m
+  f32x16 acc[NBW][MB]; // [nb][mb]: rows n, columns m
 #pragma unroll
-  for (int nb = 0; nb < 2; nb++)
+  for (int nb = 0; nb < NBW; nb++)
 #pragma unroll
-    for (int mb = 0; mb < 2; mb++)
+    for (int mb = 0; mb < MB; mb++)
 #pragma unroll
       for (int i = 0; i < 16; i++) acc[nb][mb][i] = 0.0f;
 
@@ -167,74 +191,78 @@ __global__ __launch_bounds__(256, 3) void gemm_mfma_kernel(const uint16_t *__res
     // The loads of stage kt (and of nothing later) must have landed; the barrier
     // makes every wavefront's share visible and says that everybody is done
     // with stage kt-1, which the next load overwrites.
-    if (kt + 1 < nk) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (kt + 1 < nk) {
+      if (NL == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
     __syncthreads();
     if (kt + kRing - 1 < nk) issueStage(kt + kRing - 1);
 
     const uint32_t stageBase = ldsBase + (uint32_t)((kt % kRing) * (2 * kSlice));
 #pragma unroll
-    for (int c = 0; c < 2; c++) {
-      v8 b[2], a[2];
+    for (int c = 0; c < NC; c++) {
+      v8 b[MB], a[NBW];
 #pragma unroll
-      for (int mb = 0; mb < 2; mb++)
+      for (int mb = 0; mb < MB; mb++)
         b[mb] = *reinterpret_cast<const v8 __attribute__((address_space(3))) *>(
             (const lds_u8 *)(uintptr_t)(stageBase + afrag[mb][c]));
 #pragma unroll
-      for (int nb = 0; nb < 2; nb++) {
+      for (int nb = 0; nb < NBW; nb++) {
         const lds_u8 *p = (const lds_u8 *)(uintptr_t)(stageBase + wfrag[nb]) + 16 * c * kWRow;
         const v4 lo = M::readTr(p);             // k-slots 0..3
         const v4 hi = M::readTr(p + 4 * kWRow); // k-slots 4..7
         a[nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       }
 #pragma unroll
-      for (int nb = 0; nb < 2; nb++)
+      for (int nb = 0; nb < NBW; nb++)
 #pragma unroll
-        for (int mb = 0; mb < 2; mb++) acc[nb][mb] = M::run(a[nb], b[mb], acc[nb][mb]);
+        for (int mb = 0; mb < MB; mb++) acc[nb][mb] = M::run(a[nb], b[mb], acc[nb][mb]);
     }
   }
 
   // ---- epilogue: bias, activation, residual; transpose through LDS; store ------
   __syncthreads(); // every wavefront is done reading the slices
-  uint16_t *stage = reinterpret_cast<uint16_t *>(smem) + wave * (64 * kOutStride);
-  const int mw = m0 + wm * 64, nw = n0 + wn * 64; // origin of the wavefront's quadrant
-  // All bias pieces of the quadrant first, then per 32-column block all of its
+  uint16_t *stage = reinterpret_cast<uint16_t *>(smem) + wave * (32 * MB * kOutStride);
+  const int mw = m0 + wm * (32 * MB), nw = n0 + wn * (32 * NBW); // origin of the wavefront's part
+  // All bias pieces of the part first, then per 32-column block all of its
   // residual pieces, so that the loads of a batch are in flight together.
-  v4 braw[2][4];
+  v4 braw[NBW][4];
 #pragma unroll
-  for (int nb = 0; nb < 2; nb++)
+  for (int nb = 0; nb < NBW; nb++)
 #pragma unroll
     for (int g = 0; g < 4; g++)
 #pragma unroll
       for (int i = 0; i < 4; i++) braw[nb][g][i] = M::narrow(0.0f);
   if (bias) {
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++)
+    for (int nb = 0; nb < NBW; nb++)
 #pragma unroll
       for (int g = 0; g < 4; g++) braw[nb][g] = *reinterpret_cast<const v4 *>(bias + nw + 32 * nb + 8 * g + 4 * hl);
   }
 #pragma unroll
-  for (int nb = 0; nb < 2; nb++) {
-    v4 rraw[4][2];
+  for (int nb = 0; nb < NBW; nb++) {
+    v4 rraw[4][MB];
 #pragma unroll
     for (int g = 0; g < 4; g++)
 #pragma unroll
-      for (int mb = 0; mb < 2; mb++)
+      for (int mb = 0; mb < MB; mb++)
 #pragma unroll
         for (int i = 0; i < 4; i++) rraw[g][mb][i] = M::narrow(0.0f);
     if (residual) {
 #pragma unroll
       for (int g = 0; g < 4; g++)
 #pragma unroll
-        for (int mb = 0; mb < 2; mb++)
+        for (int mb = 0; mb < MB; mb++)
           rraw[g][mb] = *reinterpret_cast<const v4 *>(residual + (size_t)(mw + 32 * mb + l32) * N + nw + 32 * nb +
                                                       8 * g + 4 * hl);
     }
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-      const int nloc = 32 * nb + 8 * g + 4 * hl; // four consecutive columns of the quadrant
+      const int nloc = 32 * nb + 8 * g + 4 * hl; // four consecutive columns of the part
 #pragma unroll
-      for (int mb = 0; mb < 2; mb++) {
+      for (int mb = 0; mb < MB; mb++) {
         const int mloc = 32 * mb + l32;
         float x[4];
 #pragma unroll
@@ -257,10 +285,11 @@ __global__ __launch_bounds__(256, 3) void gemm_mfma_kernel(const uint16_t *__res
   }
   // Each wavefront reads back only what it wrote: no block barrier needed, the
   // LDS accesses of one wavefront are ordered.
+  constexpr int kOutChunks = 4 * NBW; // 16-byte chunks per row of the part
 #pragma unroll
-  for (int it = 0; it < 8; it++) {
-    const int chunk = it * 64 + lane; // 16-byte chunk of the quadrant: 64 rows x 8
-    const int r = chunk / 8, cidx = chunk % 8;
+  for (int it = 0; it < 32 * MB * kOutChunks / 64; it++) {
+    const int chunk = it * 64 + lane;
+    const int r = chunk / kOutChunks, cidx = chunk % kOutChunks;
     // 8-byte LDS reads: the staging stride is 8-byte but not 16-byte aligned
     const u32x2 lo = *reinterpret_cast<const u32x2 *>(&stage[r * kOutStride + cidx * 8]);
     const u32x2 hi = *reinterpret_cast<const u32x2 *>(&stage[r * kOutStride + cidx * 8 + 4]);
@@ -269,22 +298,46 @@ __global__ __launch_bounds__(256, 3) void gemm_mfma_kernel(const uint16_t *__res
   }
 }
 
+template <typename T, int BK, int NB>
+void launchTile(const uint16_t *a, const uint16_t *w, const uint16_t *b, const uint16_t *r, uint16_t *o, int64_t M,
+                int64_t N, int64_t K, int act, hipStream_t stream) {
+  const int tilesN = (int)(N / (32 * NB));
+  const dim3 grid((unsigned)((M / kBM) * tilesN)), block(256);
+  if (act == ACT_GELU)
+    gemm_mfma_kernel<T, ACT_GELU, BK, NB><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+  else if (act == ACT_RELU)
+    gemm_mfma_kernel<T, ACT_RELU, BK, NB><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+  else
+    gemm_mfma_kernel<T, ACT_NONE, BK, NB><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+}
+
+// Tile width: the one under which the busiest CU carries the fewest columns
+// (tiles are dealt evenly, so that CU holds ceil(tiles / CUs) of them); 128 on
+// a tie.  Reduction step: 64 when no CU gets a second tile.
 template <typename T>
 void launch(const void *in, const void *weight, const void *bias, const void *residual, void *out, int64_t M,
             int64_t N, int64_t K, int act, hipStream_t stream) {
-  const int tilesN = (int)(N / kBN);
-  const unsigned blocks = (unsigned)((M / kBM) * tilesN);
+  const int64_t cus = numComputeUnits();
+  auto load = [&](int64_t width) -> int64_t {
+    if (N % width) return INT64_MAX;
+    const int64_t tiles = (M / kBM) * (N / width);
+    return (tiles + cus - 1) / cus * width;
+  };
+  const bool narrow = load(96) < load(128);
+  const int64_t tiles = (M / kBM) * (N / (narrow ? 96 : 128));
+  const bool deep = tiles <= cus && K % 64 == 0;
   const auto *a = static_cast<const uint16_t *>(in);
   const auto *w = static_cast<const uint16_t *>(weight);
   const auto *b = static_cast<const uint16_t *>(bias);
   const auto *r = static_cast<const uint16_t *>(residual);
   auto *o = static_cast<uint16_t *>(out);
-  if (act == ACT_GELU)
-    gemm_mfma_kernel<T, ACT_GELU><<<dim3(blocks), dim3(256), 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
-  else if (act == ACT_RELU)
-    gemm_mfma_kernel<T, ACT_RELU><<<dim3(blocks), dim3(256), 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
-  else
-    gemm_mfma_kernel<T, ACT_NONE><<<dim3(blocks), dim3(256), 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+  if (narrow) {
+    if (deep) launchTile<T, 64, 3>(a, w, b, r, o, M, N, K, act, stream);
+    else launchTile<T, 32, 3>(a, w, b, r, o, M, N, K, act, stream);
+  } else {
+    if (deep) launchTile<T, 64, 4>(a, w, b, r, o, M, N, K, act, stream);
+    else launchTile<T, 32, 4>(a, w, b, r, o, M, N, K, act, stream);
+  }
   MGPU_CHECK_LAUNCH("gemm_mfma_kernel");
 }
 
@@ -293,9 +346,9 @@ void launch(const void *in, const void *weight, const void *bias, const void *re
 bool gemmMfmaSupports(DType dt, const void *in, const void *weight, const void *bias, const void *residual,
                       const void *out, int64_t M, int64_t N, int64_t K) {
   if (dt != DType::F16 && dt != DType::BF16) return false;
-  if (M <= 0 || N <= 0 || K <= 0 || M % kBM || N % kBN || K % kBK) return false;
+  if (M <= 0 || N <= 0 || K <= 0 || M % kBM || (N % 128 && N % 96) || K % 32) return false;
   // 32-bit lane offsets inside a slice, 31-bit tile counts
-  if (K > (1 << 20) || N > (1 << 20) || (M / kBM) * (N / kBN) > 0x7fffffffLL) return false;
+  if (K > (1 << 20) || N > (1 << 20) || (M / kBM) * (N / 96) > 0x7fffffffLL) return false;
   if (!aligned16(in) || !aligned16(weight) || !aligned16(out)) return false;
   if (bias && (reinterpret_cast<uintptr_t>(bias) & 7u)) return false;
   if (residual && !aligned16(residual)) return false;

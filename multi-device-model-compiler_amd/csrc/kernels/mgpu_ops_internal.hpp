@@ -41,8 +41,8 @@ void matmulEx(DType dt, const void *input, const void *weight, const void *bias,
               const void *residual, int64_t M, int64_t N, int64_t K, bool hasBias, int act,
               bool hasResidual, hipStream_t stream);
 
-// Hand-written MFMA GEMM (gemm_mfma.hip): fp16 / bf16, M and N multiples of 128,
-// K a multiple of 32, 16-byte aligned operands; bias and residual may be null.
+// Hand-written MFMA GEMM (gemm_mfma.hip): fp16 / bf16, M a multiple of 128, N of
+// 128 or 96, K of 32, 16-byte aligned operands; bias and residual may be null.
 bool gemmMfmaSupports(DType dt, const void *in, const void *weight, const void *bias, const void *residual,
                       const void *out, int64_t M, int64_t N, int64_t K);
 void gemmMfma(DType dt, const void *in, const void *weight, const void *bias, const void *residual, void *out,

@@ -1,6 +1,7 @@
 """The hand-written MFMA GEMM (mgpuGemmMfmaF16 / BF16) against the oracle's GEMM,
-through the C ABI: every epilogue, both types, shapes from one tile and one
-reduction step up to the BERT-base layer's, and the shapes it must refuse."""
+through the C ABI: every epilogue, both types, every tile geometry, shapes from
+one tile and one reduction step up to the BERT-base layer's, and the shapes it
+must refuse."""
 import numpy as np
 import pytest
 
@@ -20,8 +21,10 @@ def spacing_tol(ref, mant_bits, floor):
     return 2.0 ** (e - mant_bits) + floor
 
 
-SHAPES = [(128, 32, 128), (128, 64, 256), (256, 96, 384), (384, 160, 128), (256, 1024, 128), (512, 768, 768),
-          (1024, 768, 3072), (4096, 768, 2304)]
+# M, K, N.  The launcher picks 128- or 96-column tiles and a reduction step of 32 or 64 from the shape (on the 256
+# CUs of the test device): both widths and both steps are in the list, N = 672 and 96 only divide by 96.
+SHAPES = [(128, 32, 128), (128, 64, 256), (256, 96, 384), (384, 160, 128), (256, 1024, 128), (256, 64, 96),
+          (128, 32, 672), (512, 768, 768), (1024, 768, 3072), (4096, 768, 2304), (4096, 64, 3072)]
 
 
 def epilogues(pkg, oracle, tb, b, tr, r):
@@ -47,7 +50,7 @@ def test_gemm_mfma_f16(pkg, gpu, oracle, rng, M, K, N):
         assert np.all(err <= spacing_tol(ref, 10, 1e-3)), (sorted(kw), err.max())
 
 
-@pytest.mark.parametrize("M,K,N", [(128, 32, 128), (256, 96, 384), (512, 768, 768)])
+@pytest.mark.parametrize("M,K,N", [(128, 32, 128), (256, 96, 384), (512, 768, 768), (4096, 64, 3072)])
 def test_gemm_mfma_bf16(pkg, gpu, oracle, rng, M, K, N):
     import torch
     mk = lambda a: torch.from_numpy(a.astype(np.float32)).to(gpu).to(torch.bfloat16)
