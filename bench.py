@@ -407,6 +407,39 @@ def main():
         fmha_case("fmha_d128_b4_s2048", "fused MHA fp16 b4 s2048 h32 d128 [long sequences, the reference layer's head size]",
                   4, 2048, 32, False, D=128)
 
+    # ---------------- GEMM with fused epilogue ---------------------------------
+    if want("gemm_ffn1_gelu"):
+        # FFN1 of the BERT-base layer: (4096 x 768) . (768 x 3072) + bias, erf-GELU.  mgpuMatmulExF16 runs whichever of
+        # the library (+ separate GELU pass) and the hand-written MFMA kernel its first-use measurement kept;
+        # mgpuGemmMfmaF16 is the hand-written kernel by itself.
+        M_, K_, N_ = 4096, 768, 3072
+        x = torch.randn((M_, K_), device=dev, generator=gen).half()
+        wt = (0.02 * torch.randn((K_, N_), device=dev, generator=gen)).half()
+        bias = (0.02 * torch.randn((N_,), device=dev, generator=gen)).half()
+        y = torch.empty((M_, N_), device=dev, dtype=torch.float16)
+
+        def gemm(fn):
+            def run(i):
+                fn(x.data_ptr(), wt.data_ptr(), bias.data_ptr(), y.data_ptr(), None, M_, N_, K_, 1, 2, 0,
+                   torch.cuda.current_stream().cuda_stream)
+            run(0)                       # first use of the shape: the selection runs here, untimed
+            torch.cuda.synchronize()
+            steps = max(20, K // 4)
+            ms = Timer(torch, use_graph=True).run(run, steps, 3)
+            check()
+            return ms * 1e3 / steps
+
+        us_auto, us_mfma = gemm(lib.mgpuMatmulExF16), gemm(lib.mgpuGemmMfmaF16)
+        flop = 2.0 * M_ * N_ * K_
+        kernels.append({"name": "gemm_ffn1_gelu",
+                        "workload": "GEMM fp16 4096x768 . 768x3072 + bias + erf-GELU (FFN1 of configs[4])",
+                        "dtype": "f16", "metric": "TFLOP/s", "value": round(flop / us_auto / 1e6, 1),
+                        "us_per_launch": round(us_auto, 2), "us_per_launch_gemm_mfma": round(us_mfma, 2),
+                        "roofline": {"bound": "mfma", "achieved": round(flop / us_auto / 1e6, 1),
+                                     "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                     "frac": round(flop / us_auto / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+                        "algorithmic_flop": flop})
+
     # ---------------- BERT-base encoder layer ----------------------------------
     if want("bert_layer"):
         B, S, d, ffn, H = 32, 128, 768, 3072, 12

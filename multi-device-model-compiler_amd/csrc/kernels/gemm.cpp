@@ -173,8 +173,8 @@ int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *resu
         libraryMs = geluMs >= 0.0f ? libraryMs + geluMs : -1.0f;
       }
       const float mfmaMs = timeLoop([&] { gemmMfma(dt, in, w, biasArg, resArg, out, M, N, K, act, s); });
-      // three per cent of margin: a tie goes to the library
-      *handWritten = libraryMs >= 0.0f && mfmaMs >= 0.0f && mfmaMs < 0.97f * libraryMs;
+      // one per cent of margin: a tie goes to the library
+      *handWritten = libraryMs >= 0.0f && mfmaMs >= 0.0f && mfmaMs < 0.99f * libraryMs;
     }
     (void)hipStreamSynchronize(s);
   }
