@@ -70,6 +70,14 @@ void mgpuLayerNormF16(const void *input, const void *gamma, const void *beta, vo
 void mgpuLayerNormBF16(const void *input, const void *gamma, const void *beta, void *output,
                        float eps, int32_t m, int32_t n, mgpuStream_t stream);
 
+/* castOut = fp16(input) and output = LayerNorm(castOut) in one pass over fp32
+ * rows: the invokeCudaCast + mgpuLayerNorm pair that opens the reference's
+ * layer (lib/Kernels/GPU/LLM.cu:37-52), with the arithmetic of the two calls
+ * (the statistics come from the rounded copy).
+ * n a multiple of 8 up to 4096 and 16-byte aligned operands, else an error. */
+void mgpuCastLayerNormF32ToF16(const float *input, const void *gamma, const void *beta, void *castOut,
+                               void *output, float eps, int32_t m, int32_t n, mgpuStream_t stream);
+
 /* output = round(fp32(input) + fp32(residual)); normed_output = LayerNorm(output)
  * with the statistics taken from the un-rounded sums.  Replaces
  * mgpuAddResidualPreLayerNorm<T> (Ops.h:63-68; LayerNorm.cu:438-466). */

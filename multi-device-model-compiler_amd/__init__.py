@@ -51,6 +51,7 @@ OPS_SIGNATURES = {
     "mgpuLayerNormF32": (None, [_c_void_p] * 4 + [_c_float, _c_int32, _c_int32, _c_void_p]),
     "mgpuLayerNormF16": (None, [_c_void_p] * 4 + [_c_float, _c_int32, _c_int32, _c_void_p]),
     "mgpuLayerNormBF16": (None, [_c_void_p] * 4 + [_c_float, _c_int32, _c_int32, _c_void_p]),
+    "mgpuCastLayerNormF32ToF16": (None, [_c_void_p] * 5 + [_c_float, _c_int32, _c_int32, _c_void_p]),
     "mgpuAddResidualPreLayerNormF32": (None, [_c_void_p] * 6 + [_c_float, _c_int32, _c_int32, _c_void_p]),
     "mgpuAddResidualPreLayerNormF16": (None, [_c_void_p] * 6 + [_c_float, _c_int32, _c_int32, _c_void_p]),
     "mgpuAddResidualPreLayerNormBF16": (None, [_c_void_p] * 6 + [_c_float, _c_int32, _c_int32, _c_void_p]),
@@ -197,6 +198,21 @@ def layer_norm(x, gamma, beta, eps: float = 1e-5, out=None, stream=None):
         _ptr(x), _ptr(gamma), _ptr(beta), _ptr(out), eps, m, n, _stream_handle(stream))
     _check(lib)
     return out
+
+
+def cast_layer_norm(x, gamma, beta, eps: float = 1e-5, stream=None):
+    """fp32 x -> (fp16 copy of x, LayerNorm of that copy in fp16), one pass."""
+    import torch
+    assert x.dtype == torch.float32
+    n = x.shape[-1]
+    m = x.numel() // n if n else 0
+    cast = torch.empty(x.shape, dtype=torch.float16, device=x.device)
+    normed = torch.empty_like(cast)
+    lib = ops()
+    lib.mgpuCastLayerNormF32ToF16(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(cast), _ptr(normed), eps, m, n,
+                                  _stream_handle(stream))
+    _check(lib)
+    return cast, normed
 
 
 def add_residual_layer_norm(x, residual, gamma, beta, eps: float = 1e-5, stream=None):

@@ -181,6 +181,13 @@ static void addResidualLN(mgpu::DType dt, const void *input, const void *residua
     mgpu::layerNorm(dt, input, residual, gamma, beta, output, normed, eps, m, n, S(stream));
   });
 }
+void mgpuCastLayerNormF32ToF16(const float *input, const void *gamma, const void *beta, void *castOut,
+                               void *output, float eps, int32_t m, int32_t n, mgpuStream_t stream) {
+  guarded([&] {
+    if (!mgpu::castLayerNormF32ToF16(input, gamma, beta, castOut, output, eps, m, n, S(stream)))
+      mgpu::fail("mgpuCastLayerNormF32ToF16: n must be a multiple of 8 up to 4096 and the operands 16-byte aligned");
+  });
+}
 void mgpuAddResidualPreLayerNormF32(const float *input, const float *residual, const float *gamma,
                                     const float *beta, float *output, float *normed_output,
                                     float eps, int32_t m, int32_t n, mgpuStream_t stream) {

@@ -131,6 +131,104 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
   }
 }
 
+// fp32 rows in, 16-bit rows out: the cast of the row (round to nearest even,
+// stored to castOut) and its LayerNorm in one pass, with the arithmetic of the
+// two-kernel sequence - the statistics and the normalisation are taken from the
+// values as rounded to T, in the lane grouping and summation order that
+// layernorm_rows_kernel uses for the same width, so the results are the same
+// bits.  Lane l of a group holds the 8-element vectors l, l + LANES, ... (two
+// 16-byte loads each).
+template <typename T, int LANES, int VPL, bool FULL>
+__global__ __launch_bounds__(256) void layernorm_cast_rows_kernel(const float *__restrict__ input,
+                                                                  const T *__restrict__ gamma,
+                                                                  const T *__restrict__ beta, T *__restrict__ castOut,
+                                                                  T *__restrict__ normed, float eps, int m, int n) {
+  using Tr = ElemTraits<T>;
+  constexpr int VEC = Tr::kVec; // 8
+  constexpr int GROUPS = 256 / LANES;
+  const int lane = threadIdx.x % LANES;
+  const int group = threadIdx.x / LANES;
+  const int nvec = n / VEC;
+  const float inv_n = 1.0f / (float)n;
+
+  const u32x4 *gv = reinterpret_cast<const u32x4 *>(gamma);
+  const u32x4 *bv = reinterpret_cast<const u32x4 *>(beta);
+  u32x4 graw[VPL], braw[VPL];
+#pragma unroll
+  for (int k = 0; k < VPL; k++) {
+    const int v = lane + k * LANES;
+    if (FULL || v < nvec) {
+      graw[k] = gv[v];
+      braw[k] = bv[v];
+    }
+  }
+
+  for (int row = blockIdx.x * GROUPS + group; row < m; row += gridDim.x * GROUPS) {
+    const u32x4 *xv = reinterpret_cast<const u32x4 *>(input + (size_t)row * n);
+    u32x4 lo[VPL], hi[VPL];
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = lane + k * LANES;
+      if (FULL || v < nvec) {
+        lo[k] = xv[2 * v];
+        hi[k] = xv[2 * v + 1];
+      }
+    }
+
+    u32x4 *cv = reinterpret_cast<u32x4 *>(castOut + (size_t)row * n);
+    float x[VPL][VEC];
+    float sum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = lane + k * LANES;
+      if (FULL || v < nvec) {
+        float a[4], b[4];
+        ElemTraits<float>::unpack(lo[k], a);
+        ElemTraits<float>::unpack(hi[k], b);
+        const float wide[VEC] = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+        const u32x4 packed = Tr::pack(wide);
+        __builtin_nontemporal_store(packed, cv + v);
+        Tr::unpack(packed, x[k]);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) sum += x[k][e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) x[k][e] = 0.0f;
+      }
+    }
+    const float mean = group_sum<LANES>(sum) * inv_n;
+
+    float sq = 0.0f;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = lane + k * LANES;
+      if (FULL || v < nvec) {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+          const float d = x[k][e] - mean;
+          sq += d * d;
+        }
+      }
+    }
+    const float var = group_sum<LANES>(sq) * inv_n;
+    const float rstd = 1.0f / sqrtf(var + eps);
+
+    u32x4 *yv = reinterpret_cast<u32x4 *>(normed + (size_t)row * n);
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = lane + k * LANES;
+      if (FULL || v < nvec) {
+        float g[VEC], b[VEC], y[VEC];
+        Tr::unpack(graw[k], g);
+        Tr::unpack(braw[k], b);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) y[e] = (x[k][e] - mean) * rstd * g[e] + b[e];
+        __builtin_nontemporal_store(Tr::pack(y), yv + v);
+      }
+    }
+  }
+}
+
 // Rows too wide for one wavefront's registers: the same scheme with a whole
 // 256-thread block per row (up to 256 x 16 vectors: 16384 fp32 or 32768
 // 16-bit elements), the two reductions finished across the 4 wavefronts
@@ -440,6 +538,42 @@ void layerNorm(DType dt, const void *input, const void *residual, const void *ga
     layerNormDispatch<bf16_t>(input, residual, gamma, beta, sumOut, normed, eps, m, n, stream);
     break;
   }
+}
+
+bool castLayerNormF32ToF16(const float *input, const void *gamma, const void *beta, void *castOut, void *normed,
+                           float eps, int m, int n, hipStream_t stream) {
+  if (m < 0 || n < 0) fail("castLayerNorm: negative shape");
+  if (m == 0 || n == 0) return true;
+  if (!input || !gamma || !beta || !castOut || !normed) fail("castLayerNorm: null pointer");
+  const int nvec = n / 8;
+  if (n % 8 || nvec > 64 * kMaxVPL || !aligned16(input) || !aligned16(gamma) || !aligned16(beta) ||
+      !aligned16(castOut) || !aligned16(normed))
+    return false;
+  // lane group and vectors per lane as layerNormTyped picks them for fp16 rows
+  const int lanes = nvec <= 16 * 4 ? 16 : nvec <= 32 * 4 ? 32 : 64;
+  const int vpl = (nvec + lanes - 1) / lanes;
+  const bool full = nvec == lanes * vpl;
+  int64_t blocks = ((int64_t)m * lanes + 255) / 256;
+  if (blocks > kMaxStreamBlocks) blocks = kMaxStreamBlocks;
+  const auto *g = static_cast<const _Float16 *>(gamma);
+  const auto *b = static_cast<const _Float16 *>(beta);
+  auto *c = static_cast<_Float16 *>(castOut);
+  auto *y = static_cast<_Float16 *>(normed);
+#define MGPU_LN_CAST(L, V)                                                                                     \
+  if (lanes == L && vpl == V) {                                                                                \
+    if (full)                                                                                                  \
+      layernorm_cast_rows_kernel<_Float16, L, V, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(      \
+          input, g, b, c, y, eps, m, n);                                                                       \
+    else                                                                                                       \
+      layernorm_cast_rows_kernel<_Float16, L, V, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(     \
+          input, g, b, c, y, eps, m, n);                                                                       \
+  }
+  MGPU_LN_CAST(16, 1) MGPU_LN_CAST(16, 2) MGPU_LN_CAST(16, 3) MGPU_LN_CAST(16, 4)
+  MGPU_LN_CAST(32, 3) MGPU_LN_CAST(32, 4)
+  MGPU_LN_CAST(64, 3) MGPU_LN_CAST(64, 4) MGPU_LN_CAST(64, 5) MGPU_LN_CAST(64, 6) MGPU_LN_CAST(64, 7) MGPU_LN_CAST(64, 8)
+#undef MGPU_LN_CAST
+  MGPU_CHECK_LAUNCH("layernorm_cast_rows_kernel");
+  return true;
 }
 
 } // namespace mgpu

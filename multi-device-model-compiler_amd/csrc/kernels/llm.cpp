@@ -2,7 +2,7 @@
 //
 // decodingContextLayer is the counterpart of mgpuLLMDecodingContextLayer
 // (lib/Kernels/GPU/LLM.cu:26-159): fp32 tensors in and out, fp16 compute,
-// weight casts on a side stream overlapped with compute through one event.
+// weight casts on a side stream overlapped with compute through events.
 // Kept from the reference: the dataflow (pre-LN, gamma = 1 / beta = 0
 // LayerNorms at eps 1e-5, packed-QKV attention, bias epilogues, residual
 // through the GEMM's C operand).  Changed on purpose:
@@ -15,6 +15,11 @@
 //    Calls on one stream are ordered by the stream; calls on different streams
 //    get different arenas.  A call made under stream capture that finds no
 //    arena large enough allocates and frees inside the capture instead;
+//  * the side stream casts all the weights as soon as the call starts, one
+//    event per GEMM, while the input cast and the first LayerNorm run on the
+//    caller's stream (the reference interleaves cast and wait per GEMM, input
+//    cast included, so the first GEMM starts two casts late); the gamma = 1 /
+//    beta = 0 vectors are written once per model width, not per call;
 //  * the side stream first waits for work already queued on the caller's
 //    stream, and the final fp16 -> fp32 cast runs after the last GEMM on the
 //    caller's stream (the reference issues it on the side stream without
@@ -35,7 +40,8 @@ namespace mgpu {
 namespace {
 
 hipStream_t copyStream = nullptr;
-hipEvent_t copyEvent = nullptr;
+constexpr int kCopyEvents = 4; // one per GEMM whose operands the side stream prepares
+hipEvent_t copyEvent[kCopyEvents] = {nullptr, nullptr, nullptr, nullptr};
 hipEvent_t forkEvent = nullptr;
 
 // Scratch memory kept per caller stream (see the header comment).
@@ -45,6 +51,29 @@ struct Scratch {
 };
 std::mutex scratchMutex;
 std::map<hipStream_t, Scratch> scratchOf;
+
+// gamma = 1, beta = 0 in fp16 for the reference layer's LayerNorms, one pair
+// per model width, written once and kept until gpuLLMOpsDeinit.
+struct Identity {
+  void *gamma = nullptr, *beta = nullptr;
+};
+std::map<int64_t, Identity> identityOf;
+
+// Null when the pair does not exist yet and cannot be made now (stream capture).
+const Identity *identityAffine(int64_t d, hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(scratchMutex);
+  auto it = identityOf.find(d);
+  if (it != identityOf.end()) return &it->second;
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) return nullptr;
+  Identity id;
+  MGPU_CHECK_HIP(hipMalloc(&id.gamma, (size_t)d * 2));
+  MGPU_CHECK_HIP(hipMalloc(&id.beta, (size_t)d * 2));
+  fillF16(id.gamma, d, 1.0f, stream);
+  fillF16(id.beta, d, 0.0f, stream);
+  MGPU_CHECK_HIP(hipStreamSynchronize(stream)); // once per width: any stream may read the pair from now on
+  return &identityOf.emplace(d, id).first->second;
+}
 
 // Bump allocator over one stream-ordered allocation; every slice is 256-byte
 // aligned so all vectorised kernels see aligned pointers.
@@ -94,7 +123,7 @@ private:
 void llmInit() {
   if (copyStream) return;
   MGPU_CHECK_HIP(hipStreamCreateWithFlags(&copyStream, hipStreamNonBlocking));
-  MGPU_CHECK_HIP(hipEventCreateWithFlags(&copyEvent, hipEventDisableTiming));
+  for (hipEvent_t &e : copyEvent) MGPU_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
   MGPU_CHECK_HIP(hipEventCreateWithFlags(&forkEvent, hipEventDisableTiming));
 }
 
@@ -106,12 +135,20 @@ void llmDeinit() {
       if (kv.second.base) (void)hipFreeAsync(kv.second.base, nullptr);
     if (!scratchOf.empty()) (void)hipStreamSynchronize(nullptr);
     scratchOf.clear();
+    for (auto &kv : identityOf) {
+      if (kv.second.gamma) (void)hipFree(kv.second.gamma);
+      if (kv.second.beta) (void)hipFree(kv.second.beta);
+    }
+    identityOf.clear();
   }
   if (copyStream) (void)hipStreamDestroy(copyStream);
-  if (copyEvent) (void)hipEventDestroy(copyEvent);
+  for (hipEvent_t &e : copyEvent) {
+    if (e) (void)hipEventDestroy(e);
+    e = nullptr;
+  }
   if (forkEvent) (void)hipEventDestroy(forkEvent);
   copyStream = nullptr;
-  copyEvent = forkEvent = nullptr;
+  forkEvent = nullptr;
 }
 
 void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *gemm_bias,
@@ -144,24 +181,44 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
   const size_t oOut = arena.reserve(M * d * h);
 
   // Fork: the side stream may not run ahead of what already sits on `stream`,
-  // the arena's allocation included.
+  // the arena's allocation included.  It then casts the weights and biases of
+  // the four GEMMs, in the order the GEMMs run, and marks each group with an
+  // event; `stream` waits for a group just before the GEMM that reads it, so the
+  // casts run under the input cast, the LayerNorms, the attention and the
+  // earlier GEMMs.
   arena.allocate(stream);
   MGPU_CHECK_HIP(hipEventRecord(forkEvent, stream));
   MGPU_CHECK_HIP(hipStreamWaitEvent(copyStream, forkEvent, 0));
-  auto sync = [&] {
-    MGPU_CHECK_HIP(hipEventRecord(copyEvent, copyStream));
-    MGPU_CHECK_HIP(hipStreamWaitEvent(stream, copyEvent, 0));
-  };
-
-  castF32ToF16(arena.at(oX), input, M * d, copyStream);
-  fillF16(arena.at(oGamma), d, 1.0f, copyStream);
-  fillF16(arena.at(oBeta), d, 0.0f, copyStream);
-  sync();
-  layerNorm(DType::F16, arena.at(oX), nullptr, arena.at(oGamma), arena.at(oBeta), nullptr,
-            arena.at(oLn), 1e-5f, (int)M, (int)d, stream);
-
   castF32ToF16(arena.at(oWqkv), qkv, d * 3 * d, copyStream);
-  sync();
+  MGPU_CHECK_HIP(hipEventRecord(copyEvent[0], copyStream));
+  castF32ToF16(arena.at(oWo), gemm_weight, d * d, copyStream);
+  castF32ToF16(arena.at(oBo), gemm_bias, d, copyStream);
+  MGPU_CHECK_HIP(hipEventRecord(copyEvent[1], copyStream));
+  castF32ToF16(arena.at(oW1), ffn1_weight, d * ffn, copyStream);
+  castF32ToF16(arena.at(oB1), ffn1_bias, ffn, copyStream);
+  MGPU_CHECK_HIP(hipEventRecord(copyEvent[2], copyStream));
+  castF32ToF16(arena.at(oW2), ffn2_weight, ffn * d, copyStream);
+  castF32ToF16(arena.at(oB2), ffn2_bias, d, copyStream);
+  MGPU_CHECK_HIP(hipEventRecord(copyEvent[3], copyStream));
+  auto join = [&](int group) { MGPU_CHECK_HIP(hipStreamWaitEvent(stream, copyEvent[group], 0)); };
+
+  const void *gamma = arena.at(oGamma), *beta = arena.at(oBeta);
+  if (const Identity *id = identityAffine(d, stream)) {
+    gamma = id->gamma;
+    beta = id->beta;
+  } else { // under capture, first use of this width: the pair lives in the arena
+    fillF16(arena.at(oGamma), d, 1.0f, stream);
+    fillF16(arena.at(oBeta), d, 0.0f, stream);
+  }
+
+  // fp16 copy of the input (the residual of the second LayerNorm) and its
+  // LayerNorm: one kernel where the width allows, else the reference's two.
+  if (!castLayerNormF32ToF16(input, gamma, beta, arena.at(oX), arena.at(oLn), 1e-5f, (int)M, (int)d, stream)) {
+    castF32ToF16(arena.at(oX), input, M * d, stream);
+    layerNorm(DType::F16, arena.at(oX), nullptr, gamma, beta, nullptr, arena.at(oLn), 1e-5f, (int)M, (int)d, stream);
+  }
+
+  join(0);
   matmulEx(DType::F16, arena.at(oLn), arena.at(oWqkv), nullptr, arena.at(oQkv), nullptr, M, 3 * d,
            d, false, ACT_NONE, false, stream);
 
@@ -169,24 +226,18 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
   fusedMHA(DType::F16, arena.at(oQkv), nullptr, arena.at(oLn), (int)batch, (int)seq_len,
            (int)heads, (int)(d_model / heads), 1.0f / sqrtf((float)(d_model / heads)), causal, stream);
 
-  castF32ToF16(arena.at(oWo), gemm_weight, d * d, copyStream);
-  castF32ToF16(arena.at(oBo), gemm_bias, d, copyStream);
-  sync();
+  join(1);
   matmulEx(DType::F16, arena.at(oLn), arena.at(oWo), arena.at(oBo), arena.at(oProj), nullptr, M, d,
            d, true, ACT_NONE, false, stream);
 
-  layerNorm(DType::F16, arena.at(oProj), arena.at(oX), arena.at(oGamma), arena.at(oBeta),
-            arena.at(oY), arena.at(oLn), 1e-5f, (int)M, (int)d, stream);
+  layerNorm(DType::F16, arena.at(oProj), arena.at(oX), gamma, beta, arena.at(oY), arena.at(oLn), 1e-5f, (int)M,
+            (int)d, stream);
 
-  castF32ToF16(arena.at(oW1), ffn1_weight, d * ffn, copyStream);
-  castF32ToF16(arena.at(oB1), ffn1_bias, ffn, copyStream);
-  sync();
+  join(2);
   matmulEx(DType::F16, arena.at(oLn), arena.at(oW1), arena.at(oB1), arena.at(oF), nullptr, M, ffn,
            d, true, relu ? ACT_RELU : ACT_GELU, false, stream);
 
-  castF32ToF16(arena.at(oW2), ffn2_weight, ffn * d, copyStream);
-  castF32ToF16(arena.at(oB2), ffn2_bias, d, copyStream);
-  sync();
+  join(3); // also the join of the fork: nothing of this call is left on the side stream after it
   matmulEx(DType::F16, arena.at(oF), arena.at(oW2), arena.at(oB2), arena.at(oOut), arena.at(oY), M,
            d, ffn, true, ACT_NONE, true, stream);
 

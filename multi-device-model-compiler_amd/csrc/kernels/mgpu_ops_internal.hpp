@@ -19,6 +19,12 @@ void layerNorm(DType dt, const void *input, const void *residual, const void *ga
                const void *beta, void *sumOut, void *normed, float eps, int m, int n,
                hipStream_t stream);
 
+// castOut = fp16(input), normed = LayerNorm(castOut) in one pass over fp32 rows
+// (n a multiple of 8 up to 4096, 16-byte aligned operands); false, with
+// nothing enqueued, for other shapes.
+bool castLayerNormF32ToF16(const float *input, const void *gamma, const void *beta, void *castOut, void *normed,
+                           float eps, int m, int n, hipStream_t stream);
+
 void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int B, int S, int H,
               int D, float scale, bool causal, hipStream_t stream);
 

@@ -146,3 +146,35 @@ def test_layernorm_in_place_and_empty(pkg, gpu, oracle, rng):
     assert_f32_close(t.cpu().numpy(), oracle.layernorm(x, g, b))
     e = torch.empty((0, 768), device=gpu)
     assert pkg.layer_norm(e, to_dev(g, gpu), to_dev(b, gpu)).shape == (0, 768)
+
+
+@pytest.mark.parametrize("m,n", [(1, 8), (5, 64), (33, 768), (100, 1000), (4096, 2048), (7, 4096), (3, 520)])
+def test_cast_layer_norm_matches_cast_then_layer_norm(pkg, gpu, oracle, rng, m, n):
+    """mgpuCastLayerNormF32ToF16 against mgpuCastF32ToF16 followed by mgpuLayerNormF16: the cast to the
+    bit, the normalised rows to one unit in the last place (the compiler may fold the final rounding
+    into the last multiply-add of one kernel and not of the other), and against the oracle like any
+    fp16 LayerNorm."""
+    import torch
+    xh = (rng.standard_normal((m, n)) * 3 + 0.5).astype(np.float32)
+    gh, bh = rng.standard_normal(n).astype(np.float16), rng.standard_normal(n).astype(np.float16)
+    x, gamma, beta = to_dev(xh, gpu), to_dev(gh, gpu), to_dev(bh, gpu)
+    cast, normed = pkg.cast_layer_norm(x, gamma, beta)
+    ref_cast = pkg.cast_f32_to_f16(x.flatten()).view(m, n)
+    ref_normed = pkg.layer_norm(ref_cast, gamma, beta)
+    assert torch.equal(cast, ref_cast)
+    bits = lambda t: t.view(torch.int16).cpu().numpy().astype(np.int32)
+    a, b = bits(normed), bits(ref_normed)
+    same_sign = (a < 0) == (b < 0)
+    assert np.all(np.where(same_sign, np.abs(a - b), np.abs(a & 0x7fff) + np.abs(b & 0x7fff)) <= 1)
+    want = oracle.layernorm(xh.astype(np.float16), gh, bh, 1e-5)
+    got = normed.cpu().numpy().astype(np.float32)
+    assert np.all(np.abs(got - want) <= 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 2.0 ** -14))) - 10) + 1e-3)
+
+
+def test_cast_layer_norm_refuses_other_widths(pkg, gpu):
+    import torch
+    for n in (12, 4104):
+        x = torch.zeros((2, n), device=gpu)
+        g = torch.zeros(n, device=gpu, dtype=torch.float16)
+        with pytest.raises(pkg.MgpuError):
+            pkg.cast_layer_norm(x, g, g)
