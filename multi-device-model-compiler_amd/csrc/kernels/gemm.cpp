@@ -149,12 +149,14 @@ int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *resu
     // The hand-written kernel on the same operands (`out` doubles as the residual).
     const void *biasArg = hasBias ? bias : nullptr, *resArg = hasResidual ? out : nullptr;
     if (bestMs >= 0.0f && gemmMfmaSupports(dt, in, w, biasArg, resArg, out, M, N, K)) {
+      // Both paths in alternating runs of twenty launches, three runs each, so that
+      // they meet the same clocks: a lone burst of a kernel that has the device to
+      // itself for a millisecond runs faster than the same kernel in a layer.
       auto timeLoop = [&](auto &&launchOnce) -> float {
         try {
-          for (int rep = 0; rep <= 20; rep++) {
-            if (rep == 1) (void)hipEventRecord(e0, s);
-            launchOnce();
-          }
+          launchOnce();
+          (void)hipEventRecord(e0, s);
+          for (int rep = 0; rep < 20; rep++) launchOnce();
         } catch (const std::exception &) {
           return -1.0f;
         }
@@ -162,19 +164,31 @@ int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *resu
         if (hipEventRecord(e1, s) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
             hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
           return -1.0f;
-        return ms / 20;
+        return ms;
       };
-      float libraryMs = bestMs;
-      if (act == ACT_GELU) {
-        const float geluMs = timeLoop([&] {
+      const float alpha1 = 1.0f, beta1 = hasResidual ? 1.0f : 0.0f;
+      auto libraryOnce = [&] {
+        if (hipblasLtMatmul(ltHandle, p.op, &alpha1, w, p.a, in, p.b, &beta1, out, p.d, out, p.d, &results[best].algo,
+                            workspace, workspaceSize, s) != HIPBLAS_STATUS_SUCCESS)
+          throw std::runtime_error("hipblasLtMatmul");
+        if (act == ACT_GELU) {
           if (dt == DType::F16) geluInPlaceF16(out, (size_t)M * N, s);
           else geluInPlaceBF16(out, (size_t)M * N, s);
-        });
-        libraryMs = geluMs >= 0.0f ? libraryMs + geluMs : -1.0f;
+        }
+      };
+      auto mfmaOnce = [&] { gemmMfma(dt, in, w, biasArg, resArg, out, M, N, K, act, s); };
+      float libraryMs = 0.0f, mfmaMs = 0.0f;
+      bool ok = true;
+      for (int round = 0; round < 3 && ok; round++) {
+        const float l = timeLoop(libraryOnce), m = timeLoop(mfmaOnce);
+        ok = l >= 0.0f && m >= 0.0f;
+        libraryMs += l;
+        mfmaMs += m;
       }
-      const float mfmaMs = timeLoop([&] { gemmMfma(dt, in, w, biasArg, resArg, out, M, N, K, act, s); });
-      // one per cent of margin: a tie goes to the library
-      *handWritten = libraryMs >= 0.0f && mfmaMs >= 0.0f && mfmaMs < 0.99f * libraryMs;
+      // The hand-written kernel has to win by 8 %: it leans harder on the L2 than the
+      // library's larger tiles do, and loses more when other streams load the memory
+      // system at the same time (the reference layer's weight casts do).
+      *handWritten = ok && mfmaMs < 0.92f * libraryMs;
     }
     (void)hipStreamSynchronize(s);
   }

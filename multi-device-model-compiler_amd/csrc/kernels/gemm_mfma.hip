@@ -21,7 +21,12 @@
 // consumed; three blocks share a CU (48 KiB of LDS, < 128 VGPRs).  When there
 // is at most one tile per CU the step is 64 instead (96 KiB of LDS): a lone
 // block cannot hide the barrier and the LDS latency of a step behind other
-// blocks, so it takes half as many, longer steps.
+// blocks, so it takes half as many, longer steps.  With several tiles per CU
+// and K a multiple of 64 the input rows are fetched for two steps at a time
+// (two buffers of 128 rows x 128 bytes, the weight slices in a ring of two):
+// a 64-byte piece of a row is half a cache line, and fetched on its own it
+// costs the whole line on the way from L2 (loads alone: 18.3 us against 21.7
+// at 4096 x 3072 x 768).
 //
 // MFMA formulation: the transposed product out^T[n, m] = W^T[n, k] . in^T[k, m],
 //   A operand = W^T: the weight slice sits in LDS row-major as in memory
@@ -59,7 +64,7 @@ __host__ __device__ constexpr int wSwz(int row) { return (row & 3) << 2; } // 16
 
 // T: element type; ACT: epilogue activation; BK: reduction step (32 or 64);
 // NB: tile width in 32-column blocks (4 or 3).
-template <typename T, int ACT, int BK, int NB>
+template <typename T, int ACT, int BK, int NB, bool PAIRED>
 __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const uint16_t *__restrict__ in,
                                                                         const uint16_t *__restrict__ weight,
                                                                         const uint16_t *__restrict__ bias,
@@ -68,7 +73,7 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
   using M = Mma<T>;
   using v8 = typename M::v8;
   using v4 = typename M::v4;
-  static_assert((BK == 32 || BK == 64) && (NB == 4 || NB == 3), "tile geometry");
+  static_assert((BK == 32 || BK == 64) && (NB == 4 || NB == 3) && (!PAIRED || BK == 32), "tile geometry");
   constexpr int kBN = 32 * NB;
   constexpr int kSlice = 256 * BK;                   // bytes of an input slice, and of a weight slice at full pitch
   constexpr int kARow = BK * 2;                      // bytes per row of the input slice: 64 / 128
@@ -81,8 +86,12 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
 
   // Ring of kRing stages, each an input slice followed by a weight slice;
   // reused as the output staging area at the end.
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[kRing * 2 * kSlice];
-  static_assert(4 * 32 * MB * kOutStride * 2 <= kRing * 2 * kSlice, "output staging must fit in the ring");
+  // PAIRED: two buffers of 16 KiB, each the input rows of two steps (128 rows of
+  // 128 bytes), then two weight slices of 8 KiB.
+  constexpr int kPairBytes = 16384, kWBase = 2 * kPairBytes;
+  constexpr int kLds = PAIRED ? kWBase + 2 * 8192 : kRing * 2 * kSlice;
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[kLds];
+  static_assert(4 * 32 * MB * kOutStride * 2 <= kLds, "output staging must fit in the ring");
 
   // Tile order.  A contiguous run of work items goes to each of the 8 XCDs
   // (consecutive block ids are dealt round-robin to the XCDs), and consecutive
@@ -128,6 +137,14 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
     if (wchunk >= 4 * NB) wchunk -= 4;
     woff[i] = (uint32_t)wrow * (uint32_t)N * 2u + (uint32_t)(wchunk * 16);
   }
+  // PAIRED: the input rows of two steps at once, 8 rows of 128 bytes per load
+  // instruction, four instructions per wavefront.
+  uint32_t aoffP[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int arow = 8 * (4 * wave + i) + lane / 8;
+    aoffP[i] = (uint32_t)arow * (uint32_t)K * 2u + (uint32_t)(((lane % 8) ^ aSwz<64>(arow)) * 16);
+  }
   // Inline assembly keeps these loads out of the compiler's wait-count
   // bookkeeping, which would otherwise wait for every load in flight before
   // any later LDS read; completion is tracked by hand (2 * NL loads per stage
@@ -151,10 +168,28 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
     }
   };
 
-  const int nk = K / BK;
+  auto issueWeights = [&](int kt) { // PAIRED: the weight slice of step kt
+    const uint32_t wdst = ldsBase + (uint32_t)(kWBase + (kt % 2) * 8192 + (2 * wave) * 1024);
+    const char *wg = wbase + (size_t)kt * 32 * N * 2;
 #pragma unroll
-  for (int t = 0; t < kRing - 1; t++)
-    if (t < nk) issueStage(t);
+    for (int i = 0; i < 2; i++) dma16(woff[i], wg, wdst + i * 1024);
+  };
+  auto issuePair = [&](int p) { // PAIRED: the input rows of steps 2p and 2p + 1
+    const uint32_t adst = ldsBase + (uint32_t)((p % 2) * kPairBytes + (4 * wave) * 1024);
+    const char *ag = abase + (size_t)p * 128;
+#pragma unroll
+    for (int i = 0; i < 4; i++) dma16(aoffP[i], ag, adst + i * 1024);
+  };
+
+  const int nk = K / BK;
+  if (PAIRED) {
+    issueWeights(0);
+    issuePair(0);
+  } else {
+#pragma unroll
+    for (int t = 0; t < kRing - 1; t++)
+      if (t < nk) issueStage(t);
+  }
 
   // ---- operand addresses inside a stage ---------------------------------------
   // in^T: lane (row 32*MB*wm + 32mb + l32, k chunk 2c + hl) reads 16 bytes.
@@ -169,13 +204,24 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
   // W^T: as a source of the transposing read, lane L of a 16-lane group g points
   // at k row 8*hl + L/4 (+ 16c, + 4 for the upper k-slots) and the four columns
   // n = 32nb + 16*(g%2) + 4*(L%4) .. +3.
-  uint32_t wfrag[NBW];
+  // PAIRED: row of a 128-byte pitch, k chunk 4 * (kt % 2) + 2c + hl of the pair's 8;
+  // the step's half is bit 2 of the chunk, i.e. bit 6 of the address, and passes
+  // through the XOR swizzle unchanged.
+  uint32_t afragP[MB][2];
+#pragma unroll
+  for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+      const int row = wm * (32 * MB) + 32 * mb + l32;
+      afragP[mb][c] = (uint32_t)(row * 128 + (((2 * c + hl) ^ aSwz<64>(row)) * 16));
+    }
+  uint32_t wfrag[NBW]; // relative to the weight slice
   {
     const int g = lane / 16, L = lane % 16, r = L % 4, j = L / 4;
 #pragma unroll
     for (int nb = 0; nb < NBW; nb++) {
       const int chunk = (4 * (NBW * wn + nb) + 2 * (g % 2) + r / 2) ^ wSwz(j);
-      wfrag[nb] = (uint32_t)(kSlice + (8 * hl + j) * kWRow + chunk * 16 + 8 * (r % 2));
+      wfrag[nb] = (uint32_t)((8 * hl + j) * kWRow + chunk * 16 + 8 * (r % 2));
     }
   }
 
@@ -188,29 +234,46 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
       for (int i = 0; i < 16; i++) acc[nb][mb][i] = 0.0f;
 
   for (int kt = 0; kt < nk; kt++) {
-    // The loads of stage kt (and of nothing later) must have landed; the barrier
-    // makes every wavefront's share visible and says that everybody is done
-    // with stage kt-1, which the next load overwrites.
-    if (kt + 1 < nk) {
-      if (NL == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    uint32_t aBase, wBase; // LDS addresses of this step's input rows and weight slice
+    if (PAIRED) {
+      // Issue order is: weights of step 1, pair 1, weights of step 2, weights of
+      // step 3, pair 2, ...  An even step needs its pair (issued two steps ago)
+      // and its weights (issued one step ago): everything in flight.  An odd step
+      // needs its weights only, issued just before the next pair: 4 loads may fly.
+      if ((kt & 1) == 0 || kt + 1 >= nk) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      __syncthreads();
+      if (kt + 1 < nk) issueWeights(kt + 1);
+      if ((kt & 1) == 0 && kt + 2 < nk) issuePair(kt / 2 + 1);
+      aBase = ldsBase + (uint32_t)(((kt / 2) % 2) * kPairBytes);
+      wBase = ldsBase + (uint32_t)(kWBase + (kt % 2) * 8192);
     } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      // The loads of stage kt (and of nothing later) must have landed; the barrier
+      // makes every wavefront's share visible and says that everybody is done
+      // with stage kt-1, which the next load overwrites.
+      if (kt + 1 < nk) {
+        if (NL == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      __syncthreads();
+      if (kt + kRing - 1 < nk) issueStage(kt + kRing - 1);
+      aBase = ldsBase + (uint32_t)((kt % kRing) * (2 * kSlice));
+      wBase = aBase + kSlice;
     }
-    __syncthreads();
-    if (kt + kRing - 1 < nk) issueStage(kt + kRing - 1);
 
-    const uint32_t stageBase = ldsBase + (uint32_t)((kt % kRing) * (2 * kSlice));
 #pragma unroll
     for (int c = 0; c < NC; c++) {
       v8 b[MB], a[NBW];
 #pragma unroll
-      for (int mb = 0; mb < MB; mb++)
-        b[mb] = *reinterpret_cast<const v8 __attribute__((address_space(3))) *>(
-            (const lds_u8 *)(uintptr_t)(stageBase + afrag[mb][c]));
+      for (int mb = 0; mb < MB; mb++) {
+        const uint32_t off = PAIRED ? (afragP[mb][c & 1] ^ ((uint32_t)(kt & 1) << 6)) : afrag[mb][c];
+        b[mb] = *reinterpret_cast<const v8 __attribute__((address_space(3))) *>((const lds_u8 *)(uintptr_t)(aBase + off));
+      }
 #pragma unroll
       for (int nb = 0; nb < NBW; nb++) {
-        const lds_u8 *p = (const lds_u8 *)(uintptr_t)(stageBase + wfrag[nb]) + 16 * c * kWRow;
+        const lds_u8 *p = (const lds_u8 *)(uintptr_t)(wBase + wfrag[nb]) + 16 * c * kWRow;
         const v4 lo = M::readTr(p);             // k-slots 0..3
         const v4 hi = M::readTr(p + 4 * kWRow); // k-slots 4..7
         a[nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -298,22 +361,23 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
   }
 }
 
-template <typename T, int BK, int NB>
+template <typename T, int BK, int NB, bool PAIRED>
 void launchTile(const uint16_t *a, const uint16_t *w, const uint16_t *b, const uint16_t *r, uint16_t *o, int64_t M,
                 int64_t N, int64_t K, int act, hipStream_t stream) {
   const int tilesN = (int)(N / (32 * NB));
   const dim3 grid((unsigned)((M / kBM) * tilesN)), block(256);
   if (act == ACT_GELU)
-    gemm_mfma_kernel<T, ACT_GELU, BK, NB><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+    gemm_mfma_kernel<T, ACT_GELU, BK, NB, PAIRED><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
   else if (act == ACT_RELU)
-    gemm_mfma_kernel<T, ACT_RELU, BK, NB><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+    gemm_mfma_kernel<T, ACT_RELU, BK, NB, PAIRED><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
   else
-    gemm_mfma_kernel<T, ACT_NONE, BK, NB><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+    gemm_mfma_kernel<T, ACT_NONE, BK, NB, PAIRED><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
 }
 
 // Tile width: the one under which the busiest CU carries the fewest columns
 // (tiles are dealt evenly, so that CU holds ceil(tiles / CUs) of them); 128 on
-// a tie.  Reduction step: 64 when no CU gets a second tile.
+// a tie.  Reduction step: 64 when no CU gets a second tile; otherwise 32, with
+// the input rows fetched in pairs of steps when K allows.
 template <typename T>
 void launch(const void *in, const void *weight, const void *bias, const void *residual, void *out, int64_t M,
             int64_t N, int64_t K, int act, hipStream_t stream) {
@@ -331,12 +395,15 @@ void launch(const void *in, const void *weight, const void *bias, const void *re
   const auto *b = static_cast<const uint16_t *>(bias);
   const auto *r = static_cast<const uint16_t *>(residual);
   auto *o = static_cast<uint16_t *>(out);
+  const bool paired = !deep && K % 64 == 0;
   if (narrow) {
-    if (deep) launchTile<T, 64, 3>(a, w, b, r, o, M, N, K, act, stream);
-    else launchTile<T, 32, 3>(a, w, b, r, o, M, N, K, act, stream);
+    if (deep) launchTile<T, 64, 3, false>(a, w, b, r, o, M, N, K, act, stream);
+    else if (paired) launchTile<T, 32, 3, true>(a, w, b, r, o, M, N, K, act, stream);
+    else launchTile<T, 32, 3, false>(a, w, b, r, o, M, N, K, act, stream);
   } else {
-    if (deep) launchTile<T, 64, 4>(a, w, b, r, o, M, N, K, act, stream);
-    else launchTile<T, 32, 4>(a, w, b, r, o, M, N, K, act, stream);
+    if (deep) launchTile<T, 64, 4, false>(a, w, b, r, o, M, N, K, act, stream);
+    else if (paired) launchTile<T, 32, 4, true>(a, w, b, r, o, M, N, K, act, stream);
+    else launchTile<T, 32, 4, false>(a, w, b, r, o, M, N, K, act, stream);
   }
   MGPU_CHECK_LAUNCH("gemm_mfma_kernel");
 }
