@@ -148,7 +148,11 @@ int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *resu
     }
     // The hand-written kernel on the same operands (`out` doubles as the residual).
     const void *biasArg = hasBias ? bias : nullptr, *resArg = hasResidual ? out : nullptr;
-    if (bestMs >= 0.0f && gemmMfmaSupports(dt, in, w, biasArg, resArg, out, M, N, K)) {
+    // Only where its short pipeline can pay: reductions up to 1024 deep, or a GELU to
+    // fuse.  On longer reductions the library's steady state (0.9-1.3 PFLOP/s) is ahead
+    // of this kernel's (0.75-1.0), and a burst of twenty launches does not always show it.
+    const bool candidate = K <= 1024 || act == ACT_GELU;
+    if (candidate && bestMs >= 0.0f && gemmMfmaSupports(dt, in, w, biasArg, resArg, out, M, N, K)) {
       // Both paths in alternating runs of twenty launches, three runs each, so that
       // they meet the same clocks: a lone burst of a kernel that has the device to
       // itself for a millisecond runs faster than the same kernel in a layer.
