@@ -130,3 +130,42 @@ def test_gelu_erfc_form_tail(pkg, gpu, oracle):
     # at most one unit in the last place of the fp16 result, subnormals included
     ulps = np.abs(got.view(np.int16).astype(np.int32) - want.view(np.int16).astype(np.int32))
     assert ulps.max() <= 1, ulps.max()
+
+
+def test_forced_kernel_choice_in_a_fresh_process(gpu):
+    """MGPU_GEMM_KERNEL=mfma / =library fix the path behind mgpuMatmulExF16; both give
+    the same matrix up to one fp16 spacing."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import sys, numpy as np, torch; sys.path.insert(0, %r)\n"
+        "import __graft_entry__ as ge\n"
+        "pkg = ge.load_package()\n"
+        "g = torch.Generator(device='cuda:0').manual_seed(3)\n"
+        "x = torch.randn((256, 256), device='cuda:0', generator=g).half()\n"
+        "w = (torch.randn((256, 384), device='cuda:0', generator=g) / 16).half()\n"
+        "b = torch.randn((384,), device='cuda:0', generator=g).half()\n"
+        "y = pkg.matmul_ex(x, w, bias=b, act=pkg.ACT_GELU)\n"
+        "np.save(sys.argv[1], y.cpu().numpy())\n" % root)
+    outs = {}
+    for mode in ("mfma", "library"):
+        path = os.path.join("/tmp", "mgpu_forced_%s_%d.npy" % (mode, os.getpid()))
+        env = dict(os.environ, MGPU_GEMM_KERNEL=mode)
+        r = subprocess.run([sys.executable, "-c", code, path], env=env, capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        outs[mode] = np.load(path).astype(np.float32)
+        os.remove(path)
+    a, b = outs["mfma"], outs["library"]
+    # the library path rounds before the GELU, the hand-written one after it: two spacings
+    assert np.all(np.abs(a - b) <= 2 * spacing_tol(b, 10, 1e-3))
+
+
+def test_gemm_mfma_refuses_a_misaligned_bias(pkg, gpu):
+    import torch
+    x = torch.zeros((128, 32), dtype=torch.float16, device=gpu)
+    w = torch.zeros((32, 128), dtype=torch.float16, device=gpu)
+    b = torch.zeros((130,), dtype=torch.float16, device=gpu)[1:129]   # 2 bytes off the 8-byte grid
+    with pytest.raises(pkg.MgpuError):
+        pkg.matmul_ex(x, w, bias=b, kernel="mfma")

@@ -86,3 +86,54 @@ def test_decoding_layer_graph(pkg, gpu):
 
     replay_against_eager(torch, st, call, lambda: x.copy_(torch.randn((B, S, d), device=gpu, generator=g)),
                          lambda: out.clone())
+
+
+def test_bert_layer_captured_on_a_stream_without_arena(pkg, gpu):
+    """First use of a stream inside a capture: the layer cannot keep an arena for the
+    stream, so it allocates and frees inside the graph; replays still match eager."""
+    import torch
+    g = torch.Generator(device=gpu).manual_seed(8)
+    B, S, d, ffn, H = 1, 64, 128, 256, 2
+    h = lambda *s: (0.05 * torch.randn(*s, device=gpu, generator=g)).half()
+    x = torch.randn((B, S, d), device=gpu, generator=g).half()
+    P = [h(d, 3 * d), h(3 * d), h(d, d), h(d), (1 + h(d).float()).half(), h(d), h(d, ffn), h(ffn), h(ffn, d), h(d),
+         (1 + h(d).float()).half(), h(d)]
+    out = torch.empty_like(x)
+    warm = torch.cuda.Stream()
+    pkg.bert_encoder_layer(x, *P, heads=H, out=out, stream=warm)   # GEMM plans exist before the capture
+    warm.synchronize()
+    ref = out.clone()
+    fresh = torch.cuda.Stream()                                     # no layer has run on this stream
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(fresh):
+        with torch.cuda.graph(graph, stream=fresh):
+            pkg.bert_encoder_layer(x, *P, heads=H, out=out, stream=fresh)
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref)
+
+
+def test_layer_arena_grows_and_is_reused(pkg, gpu, oracle):
+    """A small layer, a larger one and the small one again on one stream: the arena of
+    the stream grows once and the results do not depend on what ran before."""
+    import torch
+    g = torch.Generator(device=gpu).manual_seed(9)
+    st = torch.cuda.Stream()
+
+    def run(B, S, d, ffn, H, seed):
+        gg = torch.Generator(device=gpu).manual_seed(seed)
+        h = lambda *s: (0.05 * torch.randn(*s, device=gpu, generator=gg)).half()
+        x = torch.randn((B, S, d), device=gpu, generator=gg).half()
+        P = [h(d, 3 * d), h(3 * d), h(d, d), h(d), (1 + h(d).float()).half(), h(d), h(d, ffn), h(ffn), h(ffn, d),
+             h(d), (1 + h(d).float()).half(), h(d)]
+        out = pkg.bert_encoder_layer(x, *P, heads=H, stream=st)
+        st.synchronize()
+        return out
+
+    small1 = run(1, 32, 128, 256, 2, 100)
+    big = run(4, 128, 256, 1024, 4, 101)
+    small2 = run(1, 32, 128, 256, 2, 100)
+    assert torch.equal(small1, small2)
+    assert torch.isfinite(big.float()).all()
