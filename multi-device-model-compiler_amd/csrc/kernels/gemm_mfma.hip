@@ -19,9 +19,12 @@
 // at a 256-byte pitch) travel HBM -> LDS directly (global_load_lds, 16 bytes per
 // lane) into a ring of three stages, two steps in flight behind the one
 // consumed; three blocks share a CU (48 KiB of LDS, < 128 VGPRs).  When there
-// is at most one tile per CU the step is 64 instead (96 KiB of LDS): a lone
-// block cannot hide the barrier and the LDS latency of a step behind other
-// blocks, so it takes half as many, longer steps.  With several tiles per CU
+// is at most one tile per CU the step is 64 instead (96 KiB of LDS) and the
+// block has eight wavefronts: a lone block cannot hide the barrier and the LDS
+// latency of a step behind other blocks, so it takes half as many, longer
+// steps, and wavefronts 4-7 cover the tile like 0-3 but take the upper half of
+// every step (all eight share the loads); the two sets of accumulators meet in
+// LDS before the epilogue (4096 x 768 x 3072: 35.2 -> 30.2 us).  With several tiles per CU
 // and K a multiple of 64 the input rows are fetched for two steps at a time
 // (two buffers of 128 rows x 128 bytes, the weight slices in a ring of two):
 // a 64-byte piece of a row is half a cache line, and fetched on its own it
@@ -52,6 +55,8 @@ namespace mgpu {
 
 namespace {
 
+typedef float float4v __attribute__((ext_vector_type(4)));
+
 constexpr int kBM = 128;       // rows of an output tile
 constexpr int kRing = 3;       // LDS ring depth
 constexpr int kWRow = 256;     // LDS pitch of a weight-slice row, bytes (128 columns, of which NB * 32 are loaded)
@@ -64,8 +69,8 @@ __host__ __device__ constexpr int wSwz(int row) { return (row & 3) << 2; } // 16
 
 // T: element type; ACT: epilogue activation; BK: reduction step (32 or 64);
 // NB: tile width in 32-column blocks (4 or 3).
-template <typename T, int ACT, int BK, int NB, bool PAIRED>
-__global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const uint16_t *__restrict__ in,
+template <typename T, int ACT, int BK, int NB, bool PAIRED, bool SPLIT>
+__global__ __launch_bounds__(SPLIT ? 512 : 256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const uint16_t *__restrict__ in,
                                                                         const uint16_t *__restrict__ weight,
                                                                         const uint16_t *__restrict__ bias,
                                                                         const uint16_t *residual, uint16_t *out, int N,
@@ -73,12 +78,14 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
   using M = Mma<T>;
   using v8 = typename M::v8;
   using v4 = typename M::v4;
-  static_assert((BK == 32 || BK == 64) && (NB == 4 || NB == 3) && (!PAIRED || BK == 32), "tile geometry");
+  static_assert((BK == 32 || BK == 64) && (NB == 4 || NB == 3) && (!PAIRED || BK == 32) && (!SPLIT || BK == 64),
+                "tile geometry");
   constexpr int kBN = 32 * NB;
   constexpr int kSlice = 256 * BK;                   // bytes of an input slice, and of a weight slice at full pitch
   constexpr int kARow = BK * 2;                      // bytes per row of the input slice: 64 / 128
   constexpr int NC = BK / 16;                        // MFMA k-steps per reduction step: 2 / 4
-  constexpr int NL = BK / 16;                        // load instructions per wavefront and slice: 2 / 4
+  constexpr int NL = BK / 16 / (SPLIT ? 2 : 1);      // load instructions per wavefront and slice: 2 / 4 (2 when 8 wavefronts share them)
+  constexpr int NCW = NC / (SPLIT ? 2 : 1);          // MFMA k-steps a wavefront takes per reduction step
   constexpr int CPR = BK / 8, RPI = 64 / CPR;        // input slice: chunks per row, rows per load instruction
   constexpr int WN = NB == 4 ? 2 : 1, WM = 4 / WN;   // wavefront grid over the tile: 2 x 2 or 4 x 1
   constexpr int MB = 4 / WM, NBW = NB / WN;          // 32 x 32 accumulators per wavefront: MB x NBW = 2 x 2 or 1 x 3
@@ -113,7 +120,11 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
 
   const int tid = threadIdx.x;
   const int lane = tid % 64;
-  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  // SPLIT: eight wavefronts; 0-3 and 4-7 cover the tile in the same way and take the
+  // lower and the upper half of every reduction step, all eight share the loads.
+  const int mover = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int khalf = SPLIT ? mover / 4 : 0;
+  const int wave = SPLIT ? mover % 4 : mover;
   const int l32 = lane % 32;
   const int hl = lane / 32;
   const int wm = wave / WN, wn = wave % WN; // the wavefront's part of the tile
@@ -130,9 +141,9 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
   uint32_t aoff[NL], woff[NL];
 #pragma unroll
   for (int i = 0; i < NL; i++) {
-    const int arow = RPI * (NL * wave + i) + lane / CPR;
+    const int arow = RPI * (NL * mover + i) + lane / CPR;
     aoff[i] = (uint32_t)arow * (uint32_t)K * 2u + (uint32_t)(((lane % CPR) ^ aSwz<BK>(arow)) * 16);
-    const int wrow = 4 * (NL * wave + i) + lane / 16;
+    const int wrow = 4 * (NL * mover + i) + lane / 16;
     int wchunk = (lane % 16) ^ wSwz(wrow);
     if (wchunk >= 4 * NB) wchunk -= 4;
     woff[i] = (uint32_t)wrow * (uint32_t)N * 2u + (uint32_t)(wchunk * 16);
@@ -157,7 +168,7 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
                  : "memory");
   };
   auto issueStage = [&](int kt) {
-    const uint32_t adst = ldsBase + (uint32_t)((kt % kRing) * (2 * kSlice) + (NL * wave) * 1024);
+    const uint32_t adst = ldsBase + (uint32_t)((kt % kRing) * (2 * kSlice) + (NL * mover) * 1024);
     const uint32_t wdst = adst + kSlice;
     const char *ag = abase + (size_t)kt * kARow;
     const char *wg = wbase + (size_t)kt * BK * N * 2;
@@ -263,12 +274,15 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
       wBase = aBase + kSlice;
     }
 
+    if (SPLIT) wBase += (uint32_t)khalf * (16 * NCW * kWRow); // this half's k-steps: 32 rows further down the weight slice
 #pragma unroll
-    for (int c = 0; c < NC; c++) {
+    for (int c = 0; c < NCW; c++) {
       v8 b[MB], a[NBW];
 #pragma unroll
       for (int mb = 0; mb < MB; mb++) {
-        const uint32_t off = PAIRED ? (afragP[mb][c & 1] ^ ((uint32_t)(kt & 1) << 6)) : afrag[mb][c];
+        // SPLIT: the upper half's k-steps are chunk bit 2 of the input rows, which passes through the swizzle
+        const uint32_t off = PAIRED ? (afragP[mb][c & 1] ^ ((uint32_t)(kt & 1) << 6))
+                                    : SPLIT ? (afrag[mb][c] ^ ((uint32_t)khalf << 6)) : afrag[mb][c];
         b[mb] = *reinterpret_cast<const v8 __attribute__((address_space(3))) *>((const lds_u8 *)(uintptr_t)(aBase + off));
       }
 #pragma unroll
@@ -287,6 +301,38 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
 
   // ---- epilogue: bias, activation, residual; transpose through LDS; store ------
   __syncthreads(); // every wavefront is done reading the slices
+  if (SPLIT) {
+    // the upper half hands its accumulators to the lower half through LDS: 16
+    // bytes per lane and register group, consecutive lanes consecutive
+    float4v *red = reinterpret_cast<float4v *>(smem) + wave * (NBW * MB * 4 * 64);
+    if (khalf == 1) {
+#pragma unroll
+      for (int nb = 0; nb < NBW; nb++)
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+          for (int g = 0; g < 4; g++)
+            red[((nb * MB + mb) * 4 + g) * 64 + lane] = float4v{acc[nb][mb][4 * g], acc[nb][mb][4 * g + 1],
+                                                               acc[nb][mb][4 * g + 2], acc[nb][mb][4 * g + 3]};
+    }
+    __syncthreads();
+    if (khalf == 0) {
+#pragma unroll
+      for (int nb = 0; nb < NBW; nb++)
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            const float4v other = red[((nb * MB + mb) * 4 + g) * 64 + lane];
+            acc[nb][mb][4 * g] += other[0];
+            acc[nb][mb][4 * g + 1] += other[1];
+            acc[nb][mb][4 * g + 2] += other[2];
+            acc[nb][mb][4 * g + 3] += other[3];
+          }
+    }
+    __syncthreads(); // the staging area below overlaps what the other wavefronts have just read
+    if (khalf == 1) return;
+  }
   uint16_t *stage = reinterpret_cast<uint16_t *>(smem) + wave * (32 * MB * kOutStride);
   const int mw = m0 + wm * (32 * MB), nw = n0 + wn * (32 * NBW); // origin of the wavefront's part
   // All bias pieces of the part first, then per 32-column block all of its
@@ -361,17 +407,17 @@ __global__ __launch_bounds__(256, BK == 32 ? 3 : 1) void gemm_mfma_kernel(const 
   }
 }
 
-template <typename T, int BK, int NB, bool PAIRED>
+template <typename T, int BK, int NB, bool PAIRED, bool SPLIT = false>
 void launchTile(const uint16_t *a, const uint16_t *w, const uint16_t *b, const uint16_t *r, uint16_t *o, int64_t M,
                 int64_t N, int64_t K, int act, hipStream_t stream) {
   const int tilesN = (int)(N / (32 * NB));
-  const dim3 grid((unsigned)((M / kBM) * tilesN)), block(256);
+  const dim3 grid((unsigned)((M / kBM) * tilesN)), block(SPLIT ? 512 : 256);
   if (act == ACT_GELU)
-    gemm_mfma_kernel<T, ACT_GELU, BK, NB, PAIRED><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+    gemm_mfma_kernel<T, ACT_GELU, BK, NB, PAIRED, SPLIT><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
   else if (act == ACT_RELU)
-    gemm_mfma_kernel<T, ACT_RELU, BK, NB, PAIRED><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+    gemm_mfma_kernel<T, ACT_RELU, BK, NB, PAIRED, SPLIT><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
   else
-    gemm_mfma_kernel<T, ACT_NONE, BK, NB, PAIRED><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+    gemm_mfma_kernel<T, ACT_NONE, BK, NB, PAIRED, SPLIT><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
 }
 
 // Tile width: the one under which the busiest CU carries the fewest columns
@@ -397,11 +443,11 @@ void launch(const void *in, const void *weight, const void *bias, const void *re
   auto *o = static_cast<uint16_t *>(out);
   const bool paired = !deep && K % 64 == 0;
   if (narrow) {
-    if (deep) launchTile<T, 64, 3, false>(a, w, b, r, o, M, N, K, act, stream);
+    if (deep) launchTile<T, 64, 3, false, true>(a, w, b, r, o, M, N, K, act, stream);
     else if (paired) launchTile<T, 32, 3, true>(a, w, b, r, o, M, N, K, act, stream);
     else launchTile<T, 32, 3, false>(a, w, b, r, o, M, N, K, act, stream);
   } else {
-    if (deep) launchTile<T, 64, 4, false>(a, w, b, r, o, M, N, K, act, stream);
+    if (deep) launchTile<T, 64, 4, false, true>(a, w, b, r, o, M, N, K, act, stream);
     else if (paired) launchTile<T, 32, 4, true>(a, w, b, r, o, M, N, K, act, stream);
     else launchTile<T, 32, 4, false>(a, w, b, r, o, M, N, K, act, stream);
   }

@@ -67,7 +67,8 @@ def test_gemm_mfma_bf16(pkg, gpu, oracle, rng, M, K, N):
 def test_gemm_mfma_matches_library_path(pkg, gpu, rng):
     """The measured choice behind mgpuMatmulExF16 may be either kernel: without an
     activation both round the same fp32 sums once, so they agree to the last bit
-    wherever the two summation orders round alike, and to one spacing elsewhere."""
+    wherever the two summation orders round alike, and to one spacing elsewhere
+    (plus the fp32 noise of a 768-term sum where the terms cancel)."""
     M, K, N = 512, 768, 768
     x = rng.standard_normal((M, K)).astype(np.float16)
     w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
@@ -75,7 +76,7 @@ def test_gemm_mfma_matches_library_path(pkg, gpu, rng):
     tx, tw, tb = [to_dev(t, gpu) for t in (x, w, b)]
     a = pkg.matmul_ex(tx, tw, bias=tb).cpu().numpy().astype(np.float32)
     m = pkg.matmul_ex(tx, tw, bias=tb, kernel="mfma").cpu().numpy().astype(np.float32)
-    assert np.all(np.abs(a - m) <= spacing_tol(m, 10, 0.0))
+    assert np.all(np.abs(a - m) <= spacing_tol(m, 10, 1e-4))
     assert np.mean(a == m) > 0.99
 
 
