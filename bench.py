@@ -408,20 +408,20 @@ def main():
                   4, 2048, 32, False, D=128)
 
     # ---------------- GEMM with fused epilogue ---------------------------------
-    if want("gemm_ffn1_gelu"):
-        # FFN1 of the BERT-base layer: (4096 x 768) . (768 x 3072) + bias, erf-GELU.  mgpuMatmulExF16 runs whichever of
-        # the library (+ separate GELU pass) and the hand-written MFMA kernel its first-use measurement kept;
-        # mgpuGemmMfmaF16 is the hand-written kernel by itself.
-        M_, K_, N_ = 4096, 768, 3072
+    # The four GEMMs of the BERT-base layer at 4096 tokens.  mgpuMatmulExF16 runs whichever of the library (+ a
+    # separate GELU pass where there is one) and the hand-written MFMA kernel its first-use measurement kept;
+    # mgpuGemmMfmaF16 is the hand-written kernel by itself.
+    def gemm_case(name, workload, M_, K_, N_, act, residual):
         x = torch.randn((M_, K_), device=dev, generator=gen).half()
         wt = (0.02 * torch.randn((K_, N_), device=dev, generator=gen)).half()
         bias = (0.02 * torch.randn((N_,), device=dev, generator=gen)).half()
+        res = torch.randn((M_, N_), device=dev, generator=gen).half() if residual else None
         y = torch.empty((M_, N_), device=dev, dtype=torch.float16)
 
         def gemm(fn):
             def run(i):
-                fn(x.data_ptr(), wt.data_ptr(), bias.data_ptr(), y.data_ptr(), None, M_, N_, K_, 1, 2, 0,
-                   torch.cuda.current_stream().cuda_stream)
+                fn(x.data_ptr(), wt.data_ptr(), bias.data_ptr(), y.data_ptr(), res.data_ptr() if residual else None,
+                   M_, N_, K_, 1, act, int(residual), torch.cuda.current_stream().cuda_stream)
             run(0)                       # first use of the shape: the selection runs here, untimed
             torch.cuda.synchronize()
             steps = max(20, K // 4)
@@ -431,14 +431,23 @@ def main():
 
         us_auto, us_mfma = gemm(lib.mgpuMatmulExF16), gemm(lib.mgpuGemmMfmaF16)
         flop = 2.0 * M_ * N_ * K_
-        kernels.append({"name": "gemm_ffn1_gelu",
-                        "workload": "GEMM fp16 4096x768 . 768x3072 + bias + erf-GELU (FFN1 of configs[4])",
+        kernels.append({"name": name, "workload": workload,
                         "dtype": "f16", "metric": "TFLOP/s", "value": round(flop / us_auto / 1e6, 1),
                         "us_per_launch": round(us_auto, 2), "us_per_launch_gemm_mfma": round(us_mfma, 2),
                         "roofline": {"bound": "mfma", "achieved": round(flop / us_auto / 1e6, 1),
                                      "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                      "frac": round(flop / us_auto / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
                         "algorithmic_flop": flop})
+
+    if want("gemm_qkv"):
+        gemm_case("gemm_qkv", "GEMM fp16 4096x768 . 768x2304 + bias (QKV of configs[4])", 4096, 768, 2304, 0, False)
+    if want("gemm_proj"):
+        gemm_case("gemm_proj", "GEMM fp16 4096x768 . 768x768 + bias (projection of configs[4])", 4096, 768, 768, 0, False)
+    if want("gemm_ffn1_gelu"):
+        gemm_case("gemm_ffn1_gelu", "GEMM fp16 4096x768 . 768x3072 + bias + erf-GELU (FFN1 of configs[4])",
+                  4096, 768, 3072, 2, False)
+    if want("gemm_ffn2"):
+        gemm_case("gemm_ffn2", "GEMM fp16 4096x3072 . 3072x768 + bias (FFN2 of configs[4])", 4096, 3072, 768, 0, False)
 
     # ---------------- BERT-base encoder layer ----------------------------------
     if want("bert_layer"):
