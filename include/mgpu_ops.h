@@ -100,11 +100,26 @@ void mgpuAddResidualPreLayerNormBF16(const void *input, const void *residual, co
  * Replaces FusedMHARunnerFP16v2::setup_causal_masked_fmha + run_causal_masked_fmha
  * (3rdparty/trt_fused_multihead_attention/qkvToContext.cu:162-199,306-315) as
  * called at lib/Kernels/GPU/LLM.cu:79-81.  The reference takes b+1 prefix sums
- * (fused_multihead_attention_v2.h:63-64); this takes per-sequence lengths. */
+ * (fused_multihead_attention_v2.h:63-64); this takes per-sequence lengths over
+ * a padded [B, S] layout, the ...CuSeqlens entry points below take the prefix sums. */
 void mgpuFusedMHAF16(const void *qkv, const int32_t *seqlens, void *out, int32_t B, int32_t S,
                      int32_t H, int32_t D, float scale, int32_t causal, mgpuStream_t stream);
 void mgpuFusedMHABF16(const void *qkv, const int32_t *seqlens, void *out, int32_t B, int32_t S,
                       int32_t H, int32_t D, float scale, int32_t causal, mgpuStream_t stream);
+
+/* The same attention on the reference's own description of the sequences
+ * (fused_multihead_attention_v2.h:63-64, filled at qkvToContext.cu:162-199):
+ * cu_seqlens holds B + 1 int32 prefix sums over token rows packed back to back,
+ * qkv is [total, 3, H, D] and out [total, H*D] with total = cu_seqlens[B];
+ * sequence b owns rows cu_seqlens[b] .. cu_seqlens[b+1]-1, attends only inside
+ * itself, and max_s bounds the longest sequence (longer ones are cut to max_s
+ * keys and rows).  With cu_seqlens = {0, S, 2S, ...} this is the dense call. */
+void mgpuFusedMHAF16CuSeqlens(const void *qkv, const int32_t *cu_seqlens, void *out, int32_t B,
+                              int32_t max_s, int32_t H, int32_t D, float scale, int32_t causal,
+                              mgpuStream_t stream);
+void mgpuFusedMHABF16CuSeqlens(const void *qkv, const int32_t *cu_seqlens, void *out, int32_t B,
+                               int32_t max_s, int32_t H, int32_t D, float scale, int32_t causal,
+                               mgpuStream_t stream);
 
 /* ---- casts (Utils.h:6-8; lib/Kernels/GPU/Utils.cu:85-103) ------------- */
 void mgpuCastF32ToF16(void *dst, const float *src, size_t size, mgpuStream_t stream);

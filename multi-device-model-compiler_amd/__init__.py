@@ -57,6 +57,8 @@ OPS_SIGNATURES = {
     "mgpuAddResidualPreLayerNormBF16": (None, [_c_void_p] * 6 + [_c_float, _c_int32, _c_int32, _c_void_p]),
     "mgpuFusedMHAF16": (None, [_c_void_p] * 3 + [_c_int32] * 4 + [_c_float, _c_int32, _c_void_p]),
     "mgpuFusedMHABF16": (None, [_c_void_p] * 3 + [_c_int32] * 4 + [_c_float, _c_int32, _c_void_p]),
+    "mgpuFusedMHAF16CuSeqlens": (None, [_c_void_p] * 3 + [_c_int32] * 4 + [_c_float, _c_int32, _c_void_p]),
+    "mgpuFusedMHABF16CuSeqlens": (None, [_c_void_p] * 3 + [_c_int32] * 4 + [_c_float, _c_int32, _c_void_p]),
     "mgpuCastF32ToF16": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
     "mgpuCastF16ToF32": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
     "mgpuCastF32ToBF16": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
@@ -243,6 +245,23 @@ def fused_mha(qkv, seqlens=None, scale=None, causal: bool = False, out=None, str
     lib = ops()
     getattr(lib, "mgpuFusedMHA" + _suffix(qkv.dtype))(
         _ptr(qkv), _ptr(seqlens), _ptr(out), B, S, H, D, scale, 1 if causal else 0,
+        _stream_handle(stream))
+    _check(lib)
+    return out
+
+
+def fused_mha_cu_seqlens(qkv, cu_seqlens, max_s: int, scale=None, causal: bool = False, out=None, stream=None):
+    """qkv [total,3,H,D] fp16/bf16 packed back to back, cu_seqlens int32 [B+1] -> [total,H*D]."""
+    import torch
+    total, three, H, D = qkv.shape
+    assert three == 3 and cu_seqlens.dtype == torch.int32
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    if out is None:
+        out = torch.empty((total, H * D), dtype=qkv.dtype, device=qkv.device)
+    lib = ops()
+    getattr(lib, "mgpuFusedMHA" + _suffix(qkv.dtype) + "CuSeqlens")(
+        _ptr(qkv), _ptr(cu_seqlens), _ptr(out), cu_seqlens.numel() - 1, max_s, H, D, scale, 1 if causal else 0,
         _stream_handle(stream))
     _check(lib)
     return out

@@ -217,6 +217,19 @@ void mgpuFusedMHABF16(const void *qkv, const int32_t *seqlens, void *out, int32_
   });
 }
 
+void mgpuFusedMHAF16CuSeqlens(const void *qkv, const int32_t *cu_seqlens, void *out, int32_t B, int32_t max_s,
+                              int32_t H, int32_t D, float scale, int32_t causal, mgpuStream_t stream) {
+  guarded([&] {
+    mgpu::fusedMHACuSeqlens(mgpu::DType::F16, qkv, cu_seqlens, out, B, max_s, H, D, scale, causal != 0, S(stream));
+  });
+}
+void mgpuFusedMHABF16CuSeqlens(const void *qkv, const int32_t *cu_seqlens, void *out, int32_t B, int32_t max_s,
+                               int32_t H, int32_t D, float scale, int32_t causal, mgpuStream_t stream) {
+  guarded([&] {
+    mgpu::fusedMHACuSeqlens(mgpu::DType::BF16, qkv, cu_seqlens, out, B, max_s, H, D, scale, causal != 0, S(stream));
+  });
+}
+
 void mgpuCastF32ToF16(void *dst, const float *src, size_t size, mgpuStream_t stream) {
   guarded([&] { mgpu::castF32ToF16(dst, src, size, S(stream)); });
 }

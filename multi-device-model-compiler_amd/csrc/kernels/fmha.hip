@@ -111,6 +111,7 @@ constexpr float kSumFloor = 0.015625f;
 template <typename T, int D, int NQ, bool CAUSAL>
 __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_kernel(const uint16_t *__restrict__ qkv,
                                                               const int32_t *__restrict__ seqlens,
+                                                              const int32_t *__restrict__ cuSeqlens,
                                                               uint16_t *__restrict__ out, int S, int H,
                                                               int nQB, float scale_log2e, int pairItems) {
   using M = Mma<T>;
@@ -150,13 +151,28 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   const int l32 = lane % 32;
   const int hl = lane / 32;
 
-  int kvlen = S;
-  if (seqlens) {
+  // Two ways to say how long a sequence is.  seqlens: every sequence owns S
+  // token rows, keys beyond seqlens[b] are masked, all S query rows are
+  // produced.  cuSeqlens (b + 1 prefix sums, the reference's form): the token
+  // rows are packed back to back, sequence b owns rows cuSeqlens[b] ..
+  // cuSeqlens[b + 1] - 1 and no others exist for it; S bounds its length.
+  int kvlen = S, rows = S; // admissible keys; token rows that exist
+  size_t tok0 = (size_t)b * S;
+  if (cuSeqlens) {
+    const int first = cuSeqlens[b];
+    kvlen = cuSeqlens[b + 1] - first;
+    kvlen = kvlen < 0 ? 0 : (kvlen > S ? S : kvlen);
+    rows = kvlen;
+    tok0 = (size_t)first;
+    // Nothing to do for an empty sequence, or for a block all of whose queries lie
+    // beyond the sequence (a paired work item always holds an early block).
+    if (rows == 0 || (!paired && item * BM >= rows)) return;
+  } else if (seqlens) {
     kvlen = seqlens[b];
     kvlen = kvlen < 0 ? 0 : (kvlen > S ? S : kvlen);
   }
   const uint32_t tokBytes = (uint32_t)3 * H * kD * 2; // bytes per token row
-  const char *qbase = reinterpret_cast<const char *>(qkv) + ((size_t)b * S * 3 * H + h) * kD * 2;
+  const char *qbase = reinterpret_cast<const char *>(qkv) + (tok0 * 3 * H + h) * kD * 2;
   const char *kbase = qbase + (size_t)H * kD * 2;
   const char *vbase = qbase + (size_t)2 * H * kD * 2;
 
@@ -190,16 +206,22 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   // flight, prefetches included, before any later LDS read.  Completion is
   // tracked by hand with s_waitcnt vmcnt(n) below (4 loads per tile and wave).
   const uint32_t ldsBase = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) unsigned char *)smem);
+  // M0 is on the clobber list so that the statement counts as a definition of it
+  // (the compiler reserves M0 and notes that such a clobber is not saved and restored:
+  // nothing here needs it preserved).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
   auto dma16 = [&](uint32_t voffset, const char *sbase, uint32_t ldsAddr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(voffset), "s"(sbase), "s"(ldsAddr)
-                 : "memory");
+                 : "memory", "m0");
   };
+#pragma clang diagnostic pop
   auto issueTile = [&](int kt) {
     const uint32_t kdst = ldsBase + (uint32_t)((kt % kStages) * (2 * kTileBytes) + (2 * wave) * 1024);
     const uint32_t vdst = kdst + kTileBytes;
-    if (kt * kBN + kBN <= S) { // whole tile inside the sequence
+    if (kt * kBN + kBN <= rows) { // whole tile inside the sequence
       const char *kg = kbase + (size_t)kt * kBN * tokBytes;
       const char *vg = vbase + (size_t)kt * kBN * tokBytes;
 #pragma unroll
@@ -212,7 +234,7 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
       for (int i = 0; i < 2; i++) {
         const int row = G::RPI * (2 * wave + i) + mrow;
         int key = kt * kBN + row;
-        key = key < S ? key : S - 1;
+        key = key < rows ? key : rows - 1;
         const uint32_t rowOff = (uint32_t)key * tokBytes;
         dma16(rowOff + (mchunk ^ G::kSwz(row)) * 16, kbase, kdst + i * 1024);
         dma16(rowOff + (mchunk ^ G::vSwz(row)) * 16, vbase, vdst + i * 1024);
@@ -230,7 +252,7 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
 #pragma unroll
   for (int qi = 0; qi < NQ; qi++) {
     int row = q0 + qi * 32 + l32;
-    row = row < S ? row : S - 1;
+    row = row < rows ? row : rows - 1;
 #pragma unroll
     for (int c = 0; c < G::DC; c++)
       qf[qi][c] = *reinterpret_cast<const v8 *>(qbase + (size_t)row * tokBytes + (16 * c + 8 * hl) * 2);
@@ -427,13 +449,13 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
     const int chunk = it * 64 + lane; // 16-byte chunk index inside the wave's tile
     const int r = chunk / G::CPR, cidx = chunk % G::CPR;
     const int query = q0 + r;
-    if (query < S) {
+    if (query < rows) {
       // 8-byte LDS reads: the staging stride is 8-byte but not 16-byte aligned
       const u32x2 lo = *reinterpret_cast<const u32x2 *>(&stage[r * kOS + cidx * 8]);
       const u32x2 hi = *reinterpret_cast<const u32x2 *>(&stage[r * kOS + cidx * 8 + 4]);
       const u32x4 val = {lo[0], lo[1], hi[0], hi[1]};
       __builtin_nontemporal_store(
-          val, reinterpret_cast<u32x4 *>(out + ((size_t)b * S + query) * H * kD + (size_t)h * kD + cidx * 8));
+          val, reinterpret_cast<u32x4 *>(out + (tok0 + query) * H * kD + (size_t)h * kD + cidx * 8));
     }
   }
   // the next part's tiles land in the ring the staging area sits in
@@ -455,8 +477,8 @@ int deviceComputeUnits() {
 }
 
 template <typename T, int D, int NQ>
-void launch(const void *qkv, const int32_t *seqlens, void *out, int B, int S, int H, float scale,
-            bool causal, hipStream_t stream) {
+void launch(const void *qkv, const int32_t *seqlens, const int32_t *cuSeqlens, void *out, int B, int S, int H,
+            float scale, bool causal, hipStream_t stream) {
   constexpr int BM = 128 * NQ;
   const int nQB = (S + BM - 1) / BM;
   // Causal query blocks go in pairs of equal total work when the head dimension
@@ -469,16 +491,17 @@ void launch(const void *qkv, const int32_t *seqlens, void *out, int B, int S, in
   const auto *in = static_cast<const uint16_t *>(qkv);
   auto *o = static_cast<uint16_t *>(out);
   if (causal)
-    fmha_fwd_kernel<T, D, NQ, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, o, S, H, nQB, c, pair ? 1 : 0);
+    fmha_fwd_kernel<T, D, NQ, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0);
   else
-    fmha_fwd_kernel<T, D, NQ, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, o, S, H, nQB, c, pair ? 1 : 0);
+    fmha_fwd_kernel<T, D, NQ, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0);
   MGPU_CHECK_LAUNCH("fmha_fwd_kernel");
 }
 
 } // namespace
 
-void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int B, int S, int H,
-              int D, float scale, bool causal, hipStream_t stream) {
+namespace {
+void fusedMHAChecked(DType dt, const void *qkv, const int32_t *seqlens, const int32_t *cuSeqlens, void *out, int B,
+                     int S, int H, int D, float scale, bool causal, hipStream_t stream) {
   if (B < 0 || S < 0 || H < 0) fail("fusedMHA: negative shape");
   if (D != 64 && D != 128) fail("fusedMHA: head_dim must be 64 or 128");
   if (B == 0 || S == 0 || H == 0) return;
@@ -490,14 +513,26 @@ void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int 
   // LDS operand traffic per flop, but at 224 VGPRs only two wavefronts fit a
   // SIMD and the kernel measured slower at every shape tried.
   if (dt == DType::F16) {
-    if (D == 64) launch<_Float16, 64, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
-    else launch<_Float16, 128, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
+    if (D == 64) launch<_Float16, 64, 1>(qkv, seqlens, cuSeqlens, out, B, S, H, scale, causal, stream);
+    else launch<_Float16, 128, 1>(qkv, seqlens, cuSeqlens, out, B, S, H, scale, causal, stream);
   } else if (dt == DType::BF16) {
-    if (D == 64) launch<bf16_t, 64, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
-    else launch<bf16_t, 128, 1>(qkv, seqlens, out, B, S, H, scale, causal, stream);
+    if (D == 64) launch<bf16_t, 64, 1>(qkv, seqlens, cuSeqlens, out, B, S, H, scale, causal, stream);
+    else launch<bf16_t, 128, 1>(qkv, seqlens, cuSeqlens, out, B, S, H, scale, causal, stream);
   } else {
     fail("fusedMHA: element type must be fp16 or bf16");
   }
+}
+} // namespace
+
+void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int B, int S, int H,
+              int D, float scale, bool causal, hipStream_t stream) {
+  fusedMHAChecked(dt, qkv, seqlens, nullptr, out, B, S, H, D, scale, causal, stream);
+}
+
+void fusedMHACuSeqlens(DType dt, const void *qkv, const int32_t *cuSeqlens, void *out, int B, int maxS, int H,
+                       int D, float scale, bool causal, hipStream_t stream) {
+  if (!cuSeqlens && B > 0 && maxS > 0 && H > 0) fail("fusedMHA: cu_seqlens is null");
+  fusedMHAChecked(dt, qkv, nullptr, cuSeqlens, out, B, maxS, H, D, scale, causal, stream);
 }
 
 } // namespace mgpu

@@ -161,12 +161,18 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256, BK == 32 ? 3 : 1) void gemm_mfma
   // any later LDS read; completion is tracked by hand (2 * NL loads per stage
   // and wavefront).
   const uint32_t ldsBase = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) unsigned char *)smem);
+  // M0 is on the clobber list so that the statement counts as a definition of it
+  // (the compiler reserves M0 and notes that such a clobber is not saved and restored:
+  // nothing here needs it preserved).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
   auto dma16 = [&](uint32_t voffset, const char *sbase, uint32_t ldsAddr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(voffset), "s"(sbase), "s"(ldsAddr)
-                 : "memory");
+                 : "memory", "m0");
   };
+#pragma clang diagnostic pop
   auto issueStage = [&](int kt) {
     const uint32_t adst = ldsBase + (uint32_t)((kt % kRing) * (2 * kSlice) + (NL * mover) * 1024);
     const uint32_t wdst = adst + kSlice;

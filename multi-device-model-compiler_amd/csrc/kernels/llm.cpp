@@ -13,8 +13,11 @@
 //    cost 14 us of host time, about a tenth of a BERT-base layer): it grows to
 //    the largest layer that stream has run and is returned by gpuLLMOpsDeinit.
 //    Calls on one stream are ordered by the stream; calls on different streams
-//    get different arenas.  A call made under stream capture that finds no
-//    arena large enough allocates and frees inside the capture instead;
+//    get different arenas, side streams and events.  A call made under stream
+//    capture never touches the kept arena: it allocates and frees inside the
+//    capture, so the graph owns its temporaries and a later eager call that
+//    grows (frees and replaces) the stream's arena cannot pull memory from
+//    under a graph that is still replayed;
 //  * the side stream casts all the weights as soon as the call starts, one
 //    event per GEMM, while the input cast and the first LayerNorm run on the
 //    caller's stream (the reference interleaves cast and wait per GEMM, input
@@ -39,18 +42,38 @@ namespace mgpu {
 
 namespace {
 
-hipStream_t copyStream = nullptr;
+bool initialised = false;
 constexpr int kCopyEvents = 4; // one per GEMM whose operands the side stream prepares
-hipEvent_t copyEvent[kCopyEvents] = {nullptr, nullptr, nullptr, nullptr};
-hipEvent_t forkEvent = nullptr;
 
-// Scratch memory kept per caller stream (see the header comment).
-struct Scratch {
-  void *base = nullptr;
+// What the layers keep per caller stream between calls: the arena, and the
+// side stream with its events (two caller streams in flight at once must not
+// re-record one another's events).
+struct StreamState {
+  void *base = nullptr; // arena
   size_t bytes = 0;
+  hipStream_t side = nullptr;
+  hipEvent_t copyEvent[kCopyEvents] = {nullptr, nullptr, nullptr, nullptr};
+  hipEvent_t forkEvent = nullptr;
 };
 std::mutex scratchMutex;
-std::map<hipStream_t, Scratch> scratchOf;
+std::map<hipStream_t, StreamState> stateOf;
+
+bool isCapturing(hipStream_t s) {
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  return hipStreamIsCapturing(s, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone;
+}
+
+// The caller stream's state, with its side stream and events in place.  They
+// are created on the stream's first layer call; scratchMutex must be held.
+StreamState &sideOf(hipStream_t s) {
+  StreamState &st = stateOf[s];
+  if (!st.side) {
+    MGPU_CHECK_HIP(hipStreamCreateWithFlags(&st.side, hipStreamNonBlocking));
+    for (hipEvent_t &e : st.copyEvent) MGPU_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    MGPU_CHECK_HIP(hipEventCreateWithFlags(&st.forkEvent, hipEventDisableTiming));
+  }
+  return st;
+}
 
 // gamma = 1, beta = 0 in fp16 for the reference layer's LayerNorms, one pair
 // per model width, written once and kept until gpuLLMOpsDeinit.
@@ -64,8 +87,7 @@ const Identity *identityAffine(int64_t d, hipStream_t stream) {
   std::lock_guard<std::mutex> lock(scratchMutex);
   auto it = identityOf.find(d);
   if (it != identityOf.end()) return &it->second;
-  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) return nullptr;
+  if (isCapturing(stream)) return nullptr;
   Identity id;
   MGPU_CHECK_HIP(hipMalloc(&id.gamma, (size_t)d * 2));
   MGPU_CHECK_HIP(hipMalloc(&id.beta, (size_t)d * 2));
@@ -87,22 +109,23 @@ public:
   // Memory usable by work enqueued on `s` from here on.
   void allocate(hipStream_t s) {
     const size_t need = total_ ? total_ : 256;
+    if (isCapturing(s)) { // the graph owns its temporaries: allocated and freed inside the capture
+      MGPU_CHECK_HIP(hipMallocAsync(&base_, need, s));
+      perCall_ = true;
+      return;
+    }
     std::lock_guard<std::mutex> lock(scratchMutex);
-    Scratch &kept = scratchOf[s];
+    StreamState &kept = stateOf[s];
     if (kept.bytes >= need) {
       base_ = kept.base;
       return;
     }
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) {
-      MGPU_CHECK_HIP(hipMallocAsync(&base_, need, s)); // lives and dies inside the capture
-      perCall_ = true;
-      return;
-    }
     if (kept.base) MGPU_CHECK_HIP(hipFreeAsync(kept.base, s)); // after the work already queued on s
-    kept = Scratch{};
+    kept.base = nullptr;
+    kept.bytes = 0;
     MGPU_CHECK_HIP(hipMallocAsync(&base_, need, s));
-    kept = Scratch{base_, need};
+    kept.base = base_;
+    kept.bytes = need;
   }
   void release(hipStream_t s) {
     if (base_ && perCall_) MGPU_CHECK_HIP(hipFreeAsync(base_, s));
@@ -120,35 +143,27 @@ private:
 
 } // namespace
 
-void llmInit() {
-  if (copyStream) return;
-  MGPU_CHECK_HIP(hipStreamCreateWithFlags(&copyStream, hipStreamNonBlocking));
-  for (hipEvent_t &e : copyEvent) MGPU_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-  MGPU_CHECK_HIP(hipEventCreateWithFlags(&forkEvent, hipEventDisableTiming));
-}
+void llmInit() { initialised = true; }
 
 void llmDeinit() {
-  {
-    std::lock_guard<std::mutex> lock(scratchMutex);
-    if (!scratchOf.empty()) (void)hipDeviceSynchronize(); // the streams the arenas were ordered on may be gone
-    for (auto &kv : scratchOf)
-      if (kv.second.base) (void)hipFreeAsync(kv.second.base, nullptr);
-    if (!scratchOf.empty()) (void)hipStreamSynchronize(nullptr);
-    scratchOf.clear();
-    for (auto &kv : identityOf) {
-      if (kv.second.gamma) (void)hipFree(kv.second.gamma);
-      if (kv.second.beta) (void)hipFree(kv.second.beta);
-    }
-    identityOf.clear();
+  std::lock_guard<std::mutex> lock(scratchMutex);
+  if (!stateOf.empty()) (void)hipDeviceSynchronize(); // the streams the arenas were ordered on may be gone
+  for (auto &kv : stateOf) {
+    StreamState &st = kv.second;
+    if (st.base) (void)hipFreeAsync(st.base, nullptr);
+    if (st.side) (void)hipStreamDestroy(st.side);
+    for (hipEvent_t e : st.copyEvent)
+      if (e) (void)hipEventDestroy(e);
+    if (st.forkEvent) (void)hipEventDestroy(st.forkEvent);
   }
-  if (copyStream) (void)hipStreamDestroy(copyStream);
-  for (hipEvent_t &e : copyEvent) {
-    if (e) (void)hipEventDestroy(e);
-    e = nullptr;
+  if (!stateOf.empty()) (void)hipStreamSynchronize(nullptr);
+  stateOf.clear();
+  for (auto &kv : identityOf) {
+    if (kv.second.gamma) (void)hipFree(kv.second.gamma);
+    if (kv.second.beta) (void)hipFree(kv.second.beta);
   }
-  if (forkEvent) (void)hipEventDestroy(forkEvent);
-  copyStream = nullptr;
-  forkEvent = nullptr;
+  identityOf.clear();
+  initialised = false;
 }
 
 void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *gemm_bias,
@@ -156,7 +171,7 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
                           float *ffn2_bias, float *output, int64_t batch, int64_t seq_len,
                           int64_t d_model, int64_t ffn, int64_t heads, bool /*norm_first*/,
                           bool causal, bool relu, hipStream_t stream) {
-  if (!copyStream) fail("mgpuLLMDecodingContextLayer: gpuOpsInit() has not been called");
+  if (!initialised) fail("mgpuLLMDecodingContextLayer: gpuOpsInit() has not been called");
   if (batch < 0 || seq_len < 0 || d_model <= 0 || ffn <= 0 || heads <= 0)
     fail("mgpuLLMDecodingContextLayer: bad shape");
   if (d_model % heads || (d_model / heads != 64 && d_model / heads != 128))
@@ -187,6 +202,18 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
   // casts run under the input cast, the LayerNorms, the attention and the
   // earlier GEMMs.
   arena.allocate(stream);
+  hipStream_t copyStream = nullptr;
+  hipEvent_t forkEvent = nullptr, copyEvent[kCopyEvents];
+  {
+    // This caller stream's own side stream and events (created on its first
+    // call; under a capture that forbids creating them this fails with the
+    // runtime's message: run the layer once on the stream before capturing).
+    std::lock_guard<std::mutex> lock(scratchMutex);
+    const StreamState &st = sideOf(stream);
+    copyStream = st.side;
+    forkEvent = st.forkEvent;
+    for (int i = 0; i < kCopyEvents; i++) copyEvent[i] = st.copyEvent[i];
+  }
   MGPU_CHECK_HIP(hipEventRecord(forkEvent, stream));
   MGPU_CHECK_HIP(hipStreamWaitEvent(copyStream, forkEvent, 0));
   castF32ToF16(arena.at(oWqkv), qkv, d * 3 * d, copyStream);

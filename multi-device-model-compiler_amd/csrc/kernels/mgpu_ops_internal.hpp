@@ -28,6 +28,12 @@ bool castLayerNormF32ToF16(const float *input, const void *gamma, const void *be
 void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int B, int S, int H,
               int D, float scale, bool causal, hipStream_t stream);
 
+// The reference's form of the sequence lengths: B + 1 prefix sums over token
+// rows packed back to back (qkv [total, 3, H, D], out [total, H * D]); maxS
+// bounds the longest sequence.
+void fusedMHACuSeqlens(DType dt, const void *qkv, const int32_t *cuSeqlens, void *out, int B, int maxS, int H,
+                       int D, float scale, bool causal, hipStream_t stream);
+
 void castF32ToF16(void *dst, const float *src, size_t size, hipStream_t stream);
 void castF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream);
 void castF32ToBF16(void *dst, const float *src, size_t size, hipStream_t stream);

@@ -41,7 +41,23 @@ int main(int argc, char **argv) {
 
   if (IsPlanFile(LibPath.str())) {
     PlanModel *model = PlanModel::Load(LibPath.str(), conversion::DeviceType::GPU);
-    if (!model || !model->PrepareIO(InputData.values) || !model->Run())
+    // A rejected op or a failed runtime call leaves the output undefined: every
+    // run is followed by a look at both error slots, before anything is saved.
+    auto runChecked = [&]() -> bool {
+      if (!model->Run())
+        return false;
+      bool ok = true;
+      if (const char *err = mgpuOpsTakeLastError()) {
+        std::fprintf(stderr, "%s\n", err);
+        ok = false;
+      }
+      if (int code = mgpuRuntimeTakeLastError()) {
+        std::fprintf(stderr, "device runtime call failed with status %d\n", code);
+        ok = false;
+      }
+      return ok;
+    };
+    if (!model || !model->PrepareIO(InputData.values) || !runChecked())
       return 1;
     if (!OutputName.str().empty())
       model->SaveOutput(0, OutputName.str());
@@ -52,7 +68,7 @@ int main(int argc, char **argv) {
       float elapsed = 0;
       for (int i = 0; i < reruns; ++i) {
         mgpuEventRecord(eventBegin, stream);
-        if (!model->Run())
+        if (!runChecked())
           return 1;
         mgpuEventRecord(eventEnd, stream);
         mgpuEventSynchronize(eventEnd);
@@ -64,8 +80,6 @@ int main(int argc, char **argv) {
       std::printf("Run \t%d\ttimes\n", reruns);
       std::printf("Average time:\t%g\tseconds\n", elapsed / (reruns * 1000.0f));
     }
-    if (const char *err = mgpuOpsTakeLastError())
-      std::fprintf(stderr, "%s\n", err);
     delete model;
     gpuOpsDeinit();
     mgpuModuleUnload();

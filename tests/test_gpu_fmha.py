@@ -212,3 +212,34 @@ def test_fmha_bf16(pkg, gpu, oracle, rng):
         bits = t.view(torch.int16).cpu().numpy().view(np.uint16)
         ref = oracle.fmha(bits, lens, causal=causal, bf16=True)
         assert excess(got, ref, TOL_BF16) <= 1.0
+
+
+@pytest.mark.parametrize("lens,max_s,causal,D,dtype", [
+    ([128, 128, 128], 128, False, 64, "f16"),          # the dense call written as prefix sums
+    ([5, 0, 300, 64, 1, 129], 300, False, 64, "f16"),  # ragged, an empty sequence, tile boundaries
+    ([200, 77, 512], 512, True, 64, "f16"),            # causal: paired query blocks over packed rows
+    ([33, 250], 256, False, 128, "f16"),
+    ([100, 260], 260, True, 64, "bf16"),
+])
+def test_fmha_cu_seqlens_packed_rows(pkg, gpu, oracle, rng, lens, max_s, causal, D, dtype):
+    """The reference's own description of the batch (fused_multihead_attention_v2.h:63-64):
+    b + 1 prefix sums over token rows packed back to back.  Each sequence must come out
+    as the dense attention of that sequence alone, and no row of a neighbour is touched."""
+    import torch
+    H = 3
+    total = int(np.sum(lens))
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    qkv = rng.standard_normal((total, 3, H, D)).astype(np.float32)
+    tq = torch.from_numpy(qkv).to(gpu).to(torch.float16 if dtype == "f16" else torch.bfloat16)
+    bits = tq.view(torch.int16).cpu().numpy().view(np.uint16)  # the rounded values, as bit patterns
+    out = torch.full((total + 1, H * D), 7.0, dtype=tq.dtype, device=gpu)  # one guard row behind the batch
+    pkg.fused_mha_cu_seqlens(tq, to_dev(cu, gpu), max_s, causal=causal, out=out[:total])
+    got = out.float().cpu().numpy()
+    assert np.all(got[total] == 7.0)
+    tol = TOL_F16 if dtype == "f16" else TOL_BF16
+    for b, n in enumerate(lens):
+        if n == 0:
+            continue
+        seq = bits[cu[b]:cu[b + 1]][None]  # [1, n, 3, H, D]
+        ref = oracle.fmha(seq.view(np.float16) if dtype == "f16" else seq, None, causal=causal, bf16=dtype == "bf16")[0]
+        assert excess(got[cu[b]:cu[b + 1]], ref, tol) <= 1.0, (b, n)

@@ -137,3 +137,40 @@ def test_layer_arena_grows_and_is_reused(pkg, gpu, oracle):
     small2 = run(1, 32, 128, 256, 2, 100)
     assert torch.equal(small1, small2)
     assert torch.isfinite(big.float()).all()
+
+
+def test_captured_layer_survives_a_growing_arena(pkg, gpu):
+    """A layer captured on a stream that already keeps an arena, then a larger eager layer
+    on the same stream (the kept arena is freed and replaced), then replays: the graph
+    owns its own temporaries, so the replays still match the eager result."""
+    import torch
+    g = torch.Generator(device=gpu).manual_seed(10)
+    st = torch.cuda.Stream()
+
+    def params(d, ffn):
+        h = lambda *s: (0.05 * torch.randn(*s, device=gpu, generator=g)).half()
+        return [h(d, 3 * d), h(3 * d), h(d, d), h(d), (1 + h(d).float()).half(), h(d), h(d, ffn), h(ffn), h(ffn, d),
+                h(d), (1 + h(d).float()).half(), h(d)]
+
+    B, S, d, ffn, H = 1, 128, 128, 256, 2
+    x = torch.randn((B, S, d), device=gpu, generator=g).half()
+    P = params(d, ffn)
+    out = torch.empty_like(x)
+    pkg.bert_encoder_layer(x, *P, heads=H, out=out, stream=st)   # the stream now keeps a small arena
+    st.synchronize()
+    ref = out.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st):
+        with torch.cuda.graph(graph, stream=st):
+            pkg.bert_encoder_layer(x, *P, heads=H, out=out, stream=st)
+    xb = torch.randn((8, 128, 256), device=gpu, generator=g).half()
+    big = pkg.bert_encoder_layer(xb, *params(256, 1024), heads=4, stream=st)  # grows the arena
+    st.synchronize()
+    assert torch.isfinite(big.float()).all()
+    junk = torch.randn((64, 1024, 1024), device=gpu, generator=g)  # reuse whatever memory was returned
+    for _ in range(3):
+        out.zero_()
+        junk.mul_(1.0001)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref)
