@@ -209,6 +209,27 @@ void mgpuBertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, 
                              int64_t seq_len, int64_t d_model, int64_t feed_forward_dim,
                              int64_t head_num, float eps, mgpuStream_t stream);
 
+/* The same layer for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc);
+ * no counterpart in the reference.  Same arguments and results as
+ * mgpuBertEncoderLayerF16, but the call allocates nothing: its temporaries
+ * live in a fixed 48 MiB device array inside the library (one copy per GPU,
+ * held until the process ends) and all four GEMMs run on the hand-written MFMA
+ * kernel.  Limits, each an error reported through mgpuOpsTakeLastError():
+ *   batch*seq_len * (max(4*d_model, feed_forward_dim) + 3*d_model) * 2 bytes
+ *   must fit in 48 MiB (BERT-base (32,128,768), ffn 3072: 42 MiB);
+ *   batch*seq_len a multiple of 128, d_model and feed_forward_dim multiples
+ *   of 128 (or 96) and of 32, operands 16-byte aligned.
+ * Every call on one GPU shares that GPU's array: calls that overlap in time on
+ * different streams of one GPU race; calls on one stream are ordered. */
+void mgpuBertEncoderLayerF16NoAlloc(const void *x, const void *wqkv, const void *bqkv, const void *wo,
+                                    const void *bo, const void *gamma1, const void *beta1,
+                                    const void *w1, const void *b1, const void *w2, const void *b2,
+                                    const void *gamma2, const void *beta2, const int32_t *seqlens,
+                                    void *out, int64_t batch, int64_t seq_len, int64_t d_model,
+                                    int64_t feed_forward_dim, int64_t head_num, float eps,
+                                    mgpuStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -75,6 +75,7 @@ OPS_SIGNATURES = {
     "mgpuMatmulExF32": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuLLMDecodingContextLayer": (None, [_c_void_p] * 9 + [_c_int64] * 5 + [ctypes.c_bool] * 3 + [_c_void_p]),
     "mgpuBertEncoderLayerF16": (None, [_c_void_p] * 15 + [_c_int64] * 5 + [_c_float, _c_void_p]),
+    "mgpuBertEncoderLayerF16NoAlloc": (None, [_c_void_p] * 15 + [_c_int64] * 5 + [_c_float, _c_void_p]),
 }
 
 # mirrors include/mgpu_runtime.h
@@ -392,14 +393,17 @@ def decoding_context_layer(x, wqkv, wo, bo, w1, b1, w2, b2, heads: int, causal: 
 
 
 def bert_encoder_layer(x, wqkv, bqkv, wo, bo, g1, be1, w1, b1, w2, b2, g2, be2, heads: int,
-                       seqlens=None, eps: float = 1e-5, out=None, stream=None):
+                       seqlens=None, eps: float = 1e-5, out=None, stream=None, no_alloc: bool = False):
+    """no_alloc: the entry point whose temporaries live in the library's fixed
+    device array (the caller supplies ``out``: nothing is allocated then)."""
     import torch
     B, S, d = x.shape
     ffn = w1.shape[1]
     if out is None:
         out = torch.empty_like(x)
     lib = ops()
-    lib.mgpuBertEncoderLayerF16(_ptr(x), _ptr(wqkv), _ptr(bqkv), _ptr(wo), _ptr(bo), _ptr(g1),
+    fn = lib.mgpuBertEncoderLayerF16NoAlloc if no_alloc else lib.mgpuBertEncoderLayerF16
+    fn(_ptr(x), _ptr(wqkv), _ptr(bqkv), _ptr(wo), _ptr(bo), _ptr(g1),
                                 _ptr(be1), _ptr(w1), _ptr(b1), _ptr(w2), _ptr(b2), _ptr(g2),
                                 _ptr(be2), _ptr(seqlens), _ptr(out), B, S, d, ffn, heads, eps,
                                 _stream_handle(stream))

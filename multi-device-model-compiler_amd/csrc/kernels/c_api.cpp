@@ -40,7 +40,10 @@ inline hipStream_t S(mgpuStream_t s) { return reinterpret_cast<hipStream_t>(s); 
 
 void checkHipStatus(hipError_t status) { mgpu::checkHipStatus(status, "checkHipStatus"); }
 
-void gpuLLMOpsInit() { mgpu::llmInit(); }
+void gpuLLMOpsInit() {
+  mgpu::llmInit();
+  mgpu::noAllocInit();
+}
 void gpuLLMOpsDeinit() { mgpu::llmDeinit(); }
 
 void gpuOpsInit() {
@@ -358,6 +361,19 @@ void mgpuBertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, 
     mgpu::bertEncoderLayerF16(x, wqkv, bqkv, wo, bo, gamma1, beta1, w1, b1, w2, b2, gamma2, beta2,
                               seqlens, out, batch, seq_len, d_model, feed_forward_dim, head_num,
                               eps, S(stream));
+  });
+}
+
+void mgpuBertEncoderLayerF16NoAlloc(const void *x, const void *wqkv, const void *bqkv, const void *wo,
+                                    const void *bo, const void *gamma1, const void *beta1, const void *w1,
+                                    const void *b1, const void *w2, const void *b2, const void *gamma2,
+                                    const void *beta2, const int32_t *seqlens, void *out, int64_t batch,
+                                    int64_t seq_len, int64_t d_model, int64_t feed_forward_dim,
+                                    int64_t head_num, float eps, mgpuStream_t stream) {
+  guarded([&] {
+    mgpu::bertEncoderLayerF16NoAlloc(x, wqkv, bqkv, wo, bo, gamma1, beta1, w1, b1, w2, b2, gamma2, beta2,
+                                     seqlens, out, batch, seq_len, d_model, feed_forward_dim, head_num,
+                                     eps, S(stream));
   });
 }
 

@@ -83,6 +83,18 @@ void bertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, cons
                          int64_t S, int64_t d, int64_t ffn, int64_t H, float eps,
                          hipStream_t stream);
 
+// The same layer with every temporary in a fixed file-scope device array
+// (layer_noalloc.hip): no allocation, no library GEMM; shapes beyond the array
+// or outside the hand-written GEMM's tiling are an error.
+void noAllocInit();
+size_t noAllocScratchBytes();
+void bertEncoderLayerF16NoAlloc(const void *x, const void *wqkv, const void *bqkv, const void *wo,
+                                const void *bo, const void *gamma1, const void *beta1, const void *w1,
+                                const void *b1, const void *w2, const void *b2, const void *gamma2,
+                                const void *beta2, const int32_t *seqlens, void *out, int64_t B,
+                                int64_t S, int64_t d, int64_t ffn, int64_t H, float eps,
+                                hipStream_t stream);
+
 void geluInPlaceF16(void *data, size_t n, hipStream_t stream);
 void geluInPlaceBF16(void *data, size_t n, hipStream_t stream);
 void geluInPlaceF32(float *data, size_t n, hipStream_t stream);
