@@ -141,16 +141,16 @@ bool emitOp(Lowering &L, const DeviceOp &op, std::string &error) {
   if (n == "device.layernorm") {
     int64_t m, cols;
     rowsCols(inT(0), m, cols);
-    if (!gpu && inT(0).elem != ElemType::F32) return noCpu();
+    if (!gpu && inT(0).elem == ElemType::BF16) return noCpu();
     L.call(std::string(gpu ? "mgpuLayerNorm" : "mcpuLayerNorm") + suffixOf(inT(0).elem),
            withStream({in(0), in(1), in(2), out(0), f32(attrNumber(op, "eps", 1e-5)), i32(m), i32(cols)}));
     return true;
   }
   if (n == "device.add-residual-layernorm") {
-    if (!gpu) return noCpu();
+    if (!gpu && inT(0).elem == ElemType::BF16) return noCpu();
     int64_t m, cols;
     rowsCols(inT(0), m, cols);
-    L.call(std::string("mgpuAddResidualPreLayerNorm") + suffixOf(inT(0).elem),
+    L.call(std::string(gpu ? "mgpuAddResidualPreLayerNorm" : "mcpuAddResidualPreLayerNorm") + suffixOf(inT(0).elem),
            withStream({in(0), in(1), in(2), in(3), out(0), out(1), f32(attrNumber(op, "eps", 1e-5)), i32(m), i32(cols)}));
     return true;
   }
@@ -163,10 +163,10 @@ bool emitOp(Lowering &L, const DeviceOp &op, std::string &error) {
       L.call(gpu ? "mgpuMatmul" : "mcpuMatmul", withStream({in(0), in(1), in(2), out(0), i64(m), i64(nn), i64(k)}));
       return true;
     }
-    if (!gpu) return noCpu();
+    if (!gpu && inT(0).elem == ElemType::BF16) return noCpu();
     const std::string act = attrString(op, "act", "none");
     const int actCode = act == "relu" ? 1 : act == "gelu" ? 2 : 0;
-    L.call(std::string("mgpuMatmulEx") + suffixOf(inT(0).elem),
+    L.call(std::string(gpu ? "mgpuMatmulEx" : "mcpuMatmulEx") + suffixOf(inT(0).elem),
            withStream({in(0), in(1), in(2), out(0), in(3), i64(m), i64(nn), i64(k), i32(op.operands[2] >= 0),
                        i32(actCode), i32(op.operands[3] >= 0)}));
     return true;
@@ -202,10 +202,11 @@ bool emitOp(Lowering &L, const DeviceOp &op, std::string &error) {
     return true;
   }
   if (n == "device.cast") {
-    if (!gpu) return noCpu();
     const ElemType from = inT(0).elem, to = plan.values[op.results[0]].type.elem;
-    const char *callee = from == ElemType::F32 ? (to == ElemType::BF16 ? "mgpuCastF32ToBF16" : "mgpuCastF32ToF16")
+    if (!gpu && (from == ElemType::BF16 || to == ElemType::BF16)) return noCpu();
+    std::string callee = from == ElemType::F32 ? (to == ElemType::BF16 ? "mgpuCastF32ToBF16" : "mgpuCastF32ToF16")
                                                : (from == ElemType::BF16 ? "mgpuCastBF16ToF32" : "mgpuCastF16ToF32");
+    if (!gpu) callee[1] = 'c'; // mcpuCast...
     L.call(callee, withStream({out(0), in(0), i64(inT(0).numel())}));
     return true;
   }
@@ -219,10 +220,9 @@ bool emitOp(Lowering &L, const DeviceOp &op, std::string &error) {
     return true;
   }
   if (n == "device.multi-head-attention-layer") {
-    if (!gpu) return noCpu();
     const TensorType &x = inT(0);
-    // argument order of ConvertDeviceToLLVM.cpp:741-748
-    L.call("mgpuLLMDecodingContextLayer",
+    // argument order of ConvertDeviceToLLVM.cpp:741-748 (the CPU twin: the same without the stream)
+    L.call(gpu ? "mgpuLLMDecodingContextLayer" : "mcpuLLMDecodingContextLayer",
            withStream({in(0), in(1), in(2), in(3), in(4), in(5), in(6), in(7), out(0), i64(x.shape[0]), i64(x.shape[1]),
                        i64(x.shape[2]), i64(inT(4).shape[1]), i64((int64_t)attrNumber(op, "head_num", 0)),
                        boolean(attrBool(op, "norm_first", true)), boolean(attrBool(op, "is_casual", true)),
@@ -230,7 +230,6 @@ bool emitOp(Lowering &L, const DeviceOp &op, std::string &error) {
     return true;
   }
   if (n == "device.bert-encoder-layer") {
-    if (!gpu) return noCpu();
     const TensorType &x = inT(0);
     std::vector<CallArg> args;
     for (int i = 0; i < 14; i++) args.push_back(in(i));
@@ -238,7 +237,7 @@ bool emitOp(Lowering &L, const DeviceOp &op, std::string &error) {
     for (int64_t v : {x.shape[0], x.shape[1], x.shape[2], inT(7).shape[1], (int64_t)attrNumber(op, "head_num", 0)})
       args.push_back(i64(v));
     args.push_back(f32(attrNumber(op, "eps", 1e-5)));
-    L.call("mgpuBertEncoderLayerF16", withStream(args));
+    L.call(gpu ? "mgpuBertEncoderLayerF16" : "mcpuBertEncoderLayerF16", withStream(args));
     return true;
   }
   if (n == "gpu.launch_func") {

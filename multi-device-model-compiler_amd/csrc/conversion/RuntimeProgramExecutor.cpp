@@ -158,6 +158,27 @@ bool dispatch(Machine &m, const RuntimeCall &c) {
     ((void (*)(P, P, P, I, I, I, I, F, I))fn)(p(0), p(1), p(2), i(3), i(4), i(5), i(6), f(7), i(8));
     return true;
   }
+  if (n == "mcpuLayerNormF16") { ((void (*)(P, P, P, P, F, I, I))fn)(p(0), p(1), p(2), p(3), f(4), i(5), i(6)); return true; }
+  if (n == "mcpuAddResidualPreLayerNormF32" || n == "mcpuAddResidualPreLayerNormF16") {
+    ((void (*)(P, P, P, P, P, P, F, I, I))fn)(p(0), p(1), p(2), p(3), p(4), p(5), f(6), i(7), i(8));
+    return true;
+  }
+  if (n == "mcpuCastF32ToF16" || n == "mcpuCastF16ToF32") { ((void (*)(P, P, size_t))fn)(p(0), p(1), (size_t)l(2)); return true; }
+  if (n == "mcpuMatmulExF16" || n == "mcpuMatmulExF32") {
+    ((void (*)(P, P, P, P, P, L, L, L, I, I, I))fn)(p(0), p(1), p(2), p(3), p(4), l(5), l(6), l(7), i(8), i(9), i(10));
+    return true;
+  }
+  if (n == "mcpuLLMDecodingContextLayer") {
+    ((void (*)(P, P, P, P, P, P, P, P, P, L, L, L, L, L, bool, bool, bool))fn)(
+        p(0), p(1), p(2), p(3), p(4), p(5), p(6), p(7), p(8), l(9), l(10), l(11), l(12), l(13), b(14), b(15), b(16));
+    return true;
+  }
+  if (n == "mcpuBertEncoderLayerF16") {
+    ((void (*)(P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, L, L, L, L, L, F))fn)(
+        p(0), p(1), p(2), p(3), p(4), p(5), p(6), p(7), p(8), p(9), p(10), p(11), p(12), p(13), p(14), l(15), l(16), l(17),
+        l(18), l(19), f(20));
+    return true;
+  }
   m.error = "no prototype for callee " + n;
   return false;
 }

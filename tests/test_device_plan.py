@@ -283,7 +283,9 @@ def test_conv_pool_verifier_messages(tmp_path):
 
 
 def test_cpu_runner_reports_missing_lowerings_and_bad_files(tmp_path):
-    r = subprocess.run([CPU_RUNNER, os.path.join(PLANS, "bert_layer.plan")], capture_output=True, text=True, timeout=60)
+    bf16 = tmp_path / "bf16.plan"
+    bf16.write_text("func @main_graph(%x: 4x8xf32) -> (%y: 4x8xbf16) {\n  %y = device.cast %x : 4x8xbf16\n  return\n}\n")
+    r = subprocess.run([CPU_RUNNER, str(bf16)], capture_output=True, text=True, timeout=60)
     assert r.returncode == 1 and "has no CPU lowering" in r.stderr
     short = tmp_path / "a.dat"
     short.write_bytes(b"\0" * 12)
@@ -292,3 +294,113 @@ def test_cpu_runner_reports_missing_lowerings_and_bad_files(tmp_path):
     assert r.returncode == 1 and "Wrong File size" in r.stderr
     r = subprocess.run([CPU_RUNNER, str(tmp_path / "missing.plan")], capture_output=True, text=True, timeout=60)
     assert r.returncode == 1 and "Failed to open plan" in r.stderr
+
+
+def layer_tol(ref):
+    return 5e-3 + 4e-3 * np.abs(ref)  # fp16 output after ~6 fp16-rounded stages, see tests/test_gpu_ops_misc.py
+
+
+def test_cpu_runner_executes_the_bert_layer_plan(tmp_path, oracle):
+    """plans/bert_layer.plan (six primitive calls: matmul-ex, fused-mha, add-residual-layernorm)
+    through the CPU lowering and the CPU op library, at batch 2, against the oracle."""
+    rng = np.random.Generator(np.random.PCG64(177))
+    B, S, d, ffn, H = 2, 128, 768, 3072, 12
+    text = open(os.path.join(PLANS, "bert_layer.plan")).read().replace("32x128x", f"{B}x{S}x")
+    h16 = lambda *s: (0.02 * rng.standard_normal(s)).astype(np.float16)
+    gam = lambda: (1 + 0.02 * rng.standard_normal(d)).astype(np.float16)
+    names = ["wqkv", "bqkv", "wo", "bo", "gamma1", "beta1", "w1", "b1", "w2", "b2", "gamma2", "beta2"]
+    P = [h16(d, 3 * d), h16(3 * d), h16(d, d), h16(d), gam(), h16(d), h16(d, ffn), h16(ffn), h16(ffn, d),
+         h16(d), gam(), h16(d)]
+    for n, p in zip(names, P):
+        p.tofile(str(tmp_path / f"{n}.dat"))
+    x = rng.standard_normal((B, S, d)).astype(np.float16)
+    got, r = run_cpu_plan(tmp_path, text, [x], np.float16, (B, S, d), ("--rerun", "1"))
+    assert "Average time:\t" in r.stdout
+    ref = oracle.bert_layer_f16(x, *P, heads=H)
+    err = np.abs(got.astype(np.float32) - ref)
+    assert np.all(err <= layer_tol(ref)), err.max()
+    assert err.mean() <= 5e-4
+
+
+def test_cpu_runner_executes_the_layer_ops(tmp_path, oracle):
+    """device.multi-head-attention-layer -> mcpuLLMDecodingContextLayer (the reference's CPU
+    signature, Kernels/CPU/Ops.h:38-43) and device.bert-encoder-layer -> mcpuBertEncoderLayerF16."""
+    rng = np.random.Generator(np.random.PCG64(178))
+    B, S, d, ffn, H = 2, 64, 256, 512, 4
+    f = lambda *s, sc=0.03: (sc * rng.standard_normal(s)).astype(np.float32)
+    x = rng.standard_normal((B, S, d)).astype(np.float32)
+    W = [f(d, 3 * d), f(d, d), f(d), f(d, ffn), f(ffn), f(ffn, d), f(d)]
+    text = (f"func @main_graph(%x: {B}x{S}x{d}xf32, %qkv: {d}x{3 * d}xf32, %aw: {d}x{d}xf32, %ab: {d}xf32, "
+            f"%f1w: {d}x{ffn}xf32, %f1b: {ffn}xf32, %f2w: {ffn}x{d}xf32, %f2b: {d}xf32) -> (%y: {B}x{S}x{d}xf32) {{\n"
+            f"  %y = device.multi-head-attention-layer %x, %qkv, %aw, %ab, %f1w, %f1b, %f2w, %f2b "
+            f"{{head_num = {H}, norm_first = true, is_casual = true, act = \"relu\", batch = {B}, seq_len = {S}}} : {B}x{S}x{d}xf32\n"
+            "  return\n}\n")
+    got, _ = run_cpu_plan(tmp_path, text, [x] + W, np.float32, (B, S, d))
+    ref = oracle.decoding_context_layer(x, *W, heads=H, causal=True, act=oracle.ACT_RELU)
+    assert np.all(np.abs(got - ref) <= layer_tol(ref)), np.abs(got - ref).max()
+    assert np.array_equal(got, got.astype(np.float16).astype(np.float32))  # the final cast comes from fp16
+
+    h16 = lambda *s: (0.05 * rng.standard_normal(s)).astype(np.float16)
+    gam = lambda: (1 + 0.05 * rng.standard_normal(d)).astype(np.float16)
+    P = [h16(d, 3 * d), h16(3 * d), h16(d, d), h16(d), gam(), h16(d), h16(d, ffn), h16(ffn), h16(ffn, d),
+         h16(d), gam(), h16(d)]
+    xh = rng.standard_normal((B, S, d)).astype(np.float16)
+    lens = np.array([S, 17], np.int32)
+    shapes = [f"{d}x{3 * d}", f"{3 * d}", f"{d}x{d}", f"{d}", f"{d}", f"{d}", f"{d}x{ffn}", f"{ffn}", f"{ffn}x{d}",
+              f"{d}", f"{d}", f"{d}"]
+    args = ", ".join(f"%p{i}: {sh}xf16" for i, sh in enumerate(shapes))
+    text = (f"func @main_graph(%x: {B}x{S}x{d}xf16, {args}, %l: {B}xi32) -> (%y: {B}x{S}x{d}xf16) {{\n"
+            f"  %y = device.bert-encoder-layer %x, {', '.join(f'%p{i}' for i in range(12))}, %l {{head_num = {H}, eps = 1e-5}} "
+            f": {B}x{S}x{d}xf16\n  return\n}}\n")
+    got, _ = run_cpu_plan(tmp_path, text, [xh] + P + [lens], np.float16, (B, S, d))
+    ref = oracle.bert_layer_f16(xh, *P, heads=H, seqlens=lens)
+    err = np.abs(got.astype(np.float32) - ref)
+    assert np.all(err <= layer_tol(ref)), err.max()
+
+
+def test_cpu_twins_of_the_16_bit_entry_points(oracle, rng):
+    """mcpuLayerNormF16, mcpuAddResidualPreLayerNormF16/F32, mcpuMatmulExF16/F32 and the casts, called
+    through ctypes, against the oracle at the bounds of their GPU counterparts."""
+    import ctypes
+    lib = ctypes.CDLL(os.path.join(PKG, "lib", "libmcpu_ops.so"))
+    ptr = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    m, n = 37, 200
+    x = rng.standard_normal((m, n)).astype(np.float16)
+    res = rng.standard_normal((m, n)).astype(np.float16)
+    g = (1 + 0.1 * rng.standard_normal(n)).astype(np.float16)
+    b = (0.1 * rng.standard_normal(n)).astype(np.float16)
+    y = np.empty_like(x)
+    lib.mcpuLayerNormF16(ptr(x), ptr(g), ptr(b), ptr(y), ctypes.c_float(1e-5), m, n)
+    ref = oracle.layernorm(x, g, b)
+    ulp = lambda r: 2.0 ** (np.floor(np.log2(np.maximum(np.abs(r), 2.0 ** -14))) - 10)
+    assert np.all(np.abs(y.astype(np.float32) - ref) <= ulp(ref) + 2e-6)
+    s_out, y2 = np.empty_like(x), np.empty_like(x)
+    lib.mcpuAddResidualPreLayerNormF16(ptr(x), ptr(res), ptr(g), ptr(b), ptr(s_out), ptr(y2), ctypes.c_float(1e-5), m, n)
+    s_ref, y_ref = oracle.add_residual_layernorm(x, res, g, b)
+    assert np.array_equal(s_out.astype(np.float32), oracle.half_to_float(oracle.cast_f32_to_f16(s_ref).view(np.uint16)).reshape(m, n))
+    assert np.all(np.abs(y2.astype(np.float32) - y_ref) <= ulp(y_ref) + 2e-6)
+
+    M, K, N = 45, 96, 72
+    a = rng.standard_normal((M, K)).astype(np.float16)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    r16 = rng.standard_normal((M, N)).astype(np.float16)
+    out = np.empty((M, N), np.float16)
+    for act, residual in ((0, None), (1, None), (2, None), (0, r16)):
+        lib.mcpuMatmulExF16(ptr(a), ptr(w), ptr(bias), ptr(out), ptr(residual) if residual is not None else None,
+                            ctypes.c_int64(M), ctypes.c_int64(N), ctypes.c_int64(K), 1, act, int(residual is not None))
+        ref = oracle.gemm(a, w, bias, residual, act=act)
+        assert np.all(np.abs(out.astype(np.float32) - ref) <= ulp(ref) + 1e-5), (act, np.abs(out.astype(np.float32) - ref).max())
+    a32, w32, b32 = a.astype(np.float32), w.astype(np.float32), bias.astype(np.float32)
+    o32 = np.empty((M, N), np.float32)
+    lib.mcpuMatmulExF32(ptr(a32), ptr(w32), ptr(b32), ptr(o32), None, ctypes.c_int64(M), ctypes.c_int64(N),
+                        ctypes.c_int64(K), 1, 0, 0)
+    assert np.allclose(o32, a32.astype(np.float64) @ w32 + b32, rtol=1e-5, atol=1e-5)
+
+    f = np.concatenate([rng.standard_normal(1000) * 100, [0.0, -0.0, np.inf, -np.inf, 65504.0, 65520.0, 1e-8, 6e-8]]).astype(np.float32)
+    h = np.empty(f.shape, np.float16)
+    lib.mcpuCastF32ToF16(ptr(h), ptr(f), ctypes.c_size_t(f.size))
+    assert np.array_equal(h.view(np.uint16), oracle.cast_f32_to_f16(f).view(np.uint16))
+    back = np.empty(f.shape, np.float32)
+    lib.mcpuCastF16ToF32(ptr(back), ptr(h), ctypes.c_size_t(f.size))
+    assert np.array_equal(back.view(np.uint32), h.astype(np.float32).view(np.uint32))

@@ -85,6 +85,15 @@ def test_bert_layer_composed_from_primitive_ops(pkg, gpu, tmp_path, oracle):
     err = np.abs(got.astype(np.float32) - ref)
     assert np.all(err <= layer_tol(ref)), err.max()
     assert err.mean() <= 5e-4
+    # the same plan through the CPU lowering and the CPU op library
+    cpu_out = str(tmp_path / "out_cpu.dat")
+    r = subprocess.run([os.path.join(pkg.BIN_DIR, "multi-device-cpu-runner"), str(plan), "--data", str(tmp_path / "in0.dat"),
+                        "--out-data", cpu_out], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    cpu = np.fromfile(cpu_out, np.float16).reshape(B, S, d).astype(np.float32)
+    diff = np.abs(got.astype(np.float32) - cpu)
+    assert np.all(diff <= layer_tol(cpu)), diff.max()
+    assert diff.mean() <= 5e-4
 
 
 def test_multi_head_attention_layer_op(pkg, gpu, tmp_path, oracle):
