@@ -19,9 +19,19 @@ through enough distinct buffer sets (> 256 MiB in total) that no launch finds
 its operands in the Infinity Cache left by an earlier one; the cache-resident
 ("warm") figure is reported next to it.
 
-The CPU baseline times the oracle (a plain C port of the reference semantics)
-on the host cores for a bounded sample; it is a reported baseline, not the
-target.
+Every figure is the median of --repeats timed regions of K launches each.
+
+The CPU baseline follows the reference's CPU runner
+(tools/multi-device-cpu-runner/multi-device-cpu-runner.cpp:65-82: a clock
+around each rerun, the mean over the reruns) on this build's CPU op library
+(lib/libmcpu_ops.so, plain C++ / OpenMP, fp32 arithmetic), at one thread and
+at all host cores, on a bounded number of reruns; the reference's own compiled
+add model (oracle/_ref/libadd_ref.so, single threaded) is timed beside it when
+it has been built.  It is a reported baseline, not the target.
+
+"ceilings" reports what the device gives the simplest kernel of each kind in
+the same run: a 1 GiB copy, a copy at the headline's grid and byte count, and
+a register-fed MFMA loop with the shader clock read in the kernel.
 """
 from __future__ import annotations
 
@@ -40,22 +50,24 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 MALL_BYTES = 256 << 20
-# HBM bytes per launch, from two rocprofv3 --pmc passes over this script
-# (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0, the factors a 64 MiB device copy
-# gives for the same counters); see profiles/layernorm_f32_hbm_traffic.md for the
-# headline kernel and profiles/bench_all_configs_hbm_traffic.md for the others.
-LN_F32_TRAFFIC_BYTES = 25_250_000
-TRAFFIC_BYTES = {
-    "layernorm_f16": 12_655_000,
-    "add_f32": 14_762_000,
-    "layernorm_f32_large": 1_610_400_000,
-    "add_f32_large": 3_220_200_000,
-    "fmha_b32_s128": 25_310_000,
-    "fmha_b8_s512_masked": 31_870_000,
-    "fmha_b32_s512": 100_780_000,
-    "fmha_d128_b32_s512": 134_300_000,
-}
-# (fmha_b32_s512_causal, fmha_d128_b4_s2048, conv2d and the layers have no counter run behind them: traffic null)
+# HBM bytes per launch as counted by the hardware: profiles/hbm_traffic.json is
+# written from two rocprofv3 --pmc passes over this script (FETCH_SIZE, then
+# WRITE_SIZE, each scaled by what the same counter reads for the 64 MiB copy of
+# --copy-calibration) by tools/pmc_traffic.py and names the commit the kernels
+# were built from.  A kernel without an entry there reports traffic null.
+
+
+def load_traffic():
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            data = json.load(f)
+        return {k: v.get("bytes") for k, v in data.get("kernels", {}).items()}, data.get("commit")
+    except (OSError, ValueError):
+        return {}, None
+
+
+TRAFFIC_BYTES, TRAFFIC_COMMIT = load_traffic()
 
 
 def parse_args():
@@ -63,7 +75,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--repeats", type=int, default=7, help="timed regions of --steps launches each; the median is reported")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-ceilings", action="store_true", help="skip the copy / launch-floor / MFMA-loop probes")
     ap.add_argument("--graph", action="store_true",
                     help="time a hipGraph of K ctypes launches instead of the C++ launch loops")
     ap.add_argument("--no-graph", action="store_true", help="with --graph: enqueue the ctypes launches directly")
@@ -80,8 +94,11 @@ class Timer:
         self.torch = torch
         self.use_graph = use_graph
 
-    def run(self, fn, steps: int, warmup: int) -> float:
-        """Returns elapsed milliseconds for exactly `steps` launches."""
+    def run(self, fn, steps: int, warmup: int, repeats: int = 1) -> float:
+        """Median over `repeats` timed regions of the milliseconds for exactly `steps` launches."""
+        return float(np.median([self.run_once(fn, steps, warmup) for _ in range(max(1, repeats))]))
+
+    def run_once(self, fn, steps: int, warmup: int) -> float:
         torch = self.torch
         stream = torch.cuda.Stream()
         with torch.cuda.stream(stream):
@@ -167,6 +184,165 @@ def hbm_entry(name, workload, dtype, bytes_per_launch, ms, steps, warm_ms=None):
     return e
 
 
+
+def cpu_model_name() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baselines(pkg, m, n, ln_bytes) -> dict:
+    """Times the CPU op library the way the reference's CPU runner times a model
+    (multi-device-cpu-runner.cpp:65-82: one untimed run, then a clock around
+    each rerun, mean over the reruns), at one thread and at all host cores, for
+    add, LayerNorm fp32, attention b32 s128 and the BERT-base layer.  The number
+    of reruns is bounded by time so the whole leg stays near 25 s."""
+    lib = ctypes.CDLL(os.path.join(pkg.LIB_DIR, "libmcpu_ops.so"))
+    lib.mcpuGetNumThreads.restype = ctypes.c_int32
+    all_threads = min(int(lib.mcpuGetNumThreads()), len(os.sched_getaffinity(0)))
+    model = cpu_model_name()
+    rng = np.random.default_rng(20241)
+    P = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+
+    def reruns(fn, budget_s, max_runs):
+        fn()  # the model's first run, untimed like the runner's
+        times = []
+        t_end = time.perf_counter() + budget_s
+        while len(times) < max_runs and (len(times) < 2 or time.perf_counter() < t_end):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        return sum(times) / len(times), len(times)
+
+    def both(fn, budget_s, max_runs, to_value, unit, what):
+        res = {}
+        for threads in (all_threads, 1):
+            lib.mcpuSetNumThreads(threads)
+            sec, runs = reruns(fn, budget_s, max_runs)
+            res[threads] = (to_value(sec), sec, runs)
+        lib.mcpuSetNumThreads(all_threads)
+        v, sec, runs = res[all_threads]
+        v1, sec1, runs1 = res[1]
+        return {"value": round(v, 3), "unit": unit, "cores": all_threads, "threads": all_threads, "cpu_model": model,
+                "kind": "port", "seconds_per_run": round(sec, 6),
+                "single_thread": {"value": round(v1, 3), "unit": unit, "threads": 1, "seconds_per_run": round(sec1, 6),
+                                  "reruns": runs1},
+                "sample": f"{what}: mean of {runs} reruns of the entry point of lib/libmcpu_ops.so (fp32 arithmetic, OpenMP) "
+                          f"with a clock around each, as multi-device-cpu-runner --rerun does; {runs1} reruns at one thread"}
+
+    out = {}
+    x = rng.standard_normal((m, n)).astype(np.float32)
+    g = (1 + 0.02 * rng.standard_normal(n)).astype(np.float32)
+    b = (0.02 * rng.standard_normal(n)).astype(np.float32)
+    y = np.empty_like(x)
+    out["layernorm_f32"] = both(lambda: lib.mcpuLayerNormF32(P(x), P(g), P(b), P(y), ctypes.c_float(1e-5), m, n),
+                                1.0, 2000, lambda s: ln_bytes / s / 1e9, "GB/s", f"LayerNorm fp32 ({m},{n})")
+
+    ne = 3 * 640 * 640
+    a1 = rng.uniform(-1, 1, ne).astype(np.float32)
+    b1 = rng.uniform(-1, 1, ne).astype(np.float32)
+    c1 = np.empty_like(a1)
+    out["add_f32"] = both(lambda: lib.mcpuAddF32(P(a1), P(b1), P(c1), ctypes.c_int64(ne)), 1.0, 2000,
+                          lambda s: 3 * ne * 4 / s / 1e9, "GB/s", "add fp32 (3,640,640)")
+    # the reference's own compiled add model (examples/add.ll through llc + gcc, built by
+    # oracle/Makefile where the reference checkout exists): single threaded
+    import __graft_entry__ as ge
+    oracle = ge.load_oracle()
+    if oracle.ref_add_available():
+        times = oracle.ref_add_seconds(a1.reshape(3, 640, 640), b1.reshape(3, 640, 640), 100)
+        sec = sum(times) / len(times)
+        out["add_f32"]["reference_model"] = {
+            "value": round(3 * ne * 4 / sec / 1e9, 3), "unit": "GB/s", "threads": 1, "cores": 1, "kind": "reference",
+            "cpu_model": model, "seconds_per_run": round(sec, 6),
+            "sample": f"mean of {len(times)} reruns of _mlir_ciface_main_graph of the reference's examples/add.ll "
+                      "(oracle/_ref/libadd_ref.so), the model's malloc of its 4.9 MB output inside the clock as in "
+                      "multi-device-cpu-runner"}
+
+    B, S, H, D = 32, 128, 12, 64
+    qkv = (rng.standard_normal((B, S, 3, H, D)) / 8).astype(np.float16)
+    o = np.empty((B, S, H * D), np.float16)
+    flop = 4.0 * B * H * S * S * D
+    out["fmha_b32_s128"] = both(lambda: lib.mcpuFusedMHAF16(P(qkv), None, P(o), B, S, H, D, ctypes.c_float(0.125), 0),
+                                2.5, 50, lambda s: flop / s / 1e12, "TFLOP/s", "fused MHA fp16 b32 s128 h12 d64")
+
+    d, ffn = 768, 3072
+    h16 = lambda *sh: (0.02 * rng.standard_normal(sh)).astype(np.float16)
+    gam = lambda: (1 + 0.02 * rng.standard_normal(d)).astype(np.float16)
+    xb = rng.standard_normal((B, S, d)).astype(np.float16)
+    W = [h16(d, 3 * d), h16(3 * d), h16(d, d), h16(d), gam(), h16(d), h16(d, ffn), h16(ffn), h16(ffn, d), h16(d), gam(), h16(d)]
+    ob = np.empty_like(xb)
+    i64 = ctypes.c_int64
+    out["bert_layer"] = both(lambda: lib.mcpuBertEncoderLayerF16(P(xb), *[P(w) for w in W], None, P(ob), i64(B), i64(S), i64(d),
+                                                                  i64(ffn), i64(H), ctypes.c_float(1e-5)),
+                             4.0, 10, lambda s: s * 1e6, "us", "BERT-base encoder layer fp16 (32,128,768)")
+    return out
+
+
+def measure_ceilings(torch, loops, dev, gen, sp, ptrs, repeats) -> dict:
+    """A 1 GiB copy, a copy with the headline's grid and bytes (cold and cache
+    resident), and the register-fed MFMA loop at 1-4 wavefronts per SIMD."""
+    def med(call):
+        t = [call() for _ in range(repeats)]
+        return float(np.median(t)) if min(t) >= 0 else None
+
+    res = {}
+    big = 1 << 30
+    src = torch.empty(big, dtype=torch.uint8, device=dev).random_(generator=gen)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    ms = med(lambda: loops.mgpuProbeCopy(ptrs([src]), ptrs([dst]), 1, ctypes.c_size_t(big), 10, 2, sp))
+    if ms:
+        res["copy_1GiB"] = {"GB/s": round(2 * big * 10 / ms / 1e6, 1), "us_per_launch": round(ms * 100, 1),
+                            "what": "one 16-byte vector per lane, one block per 256 vectors, 1 GiB read + 1 GiB written"}
+    del src, dst
+    half = 32 * 128 * 768 * 4  # bytes read (and written) by the headline LayerNorm
+    nsets = rotating_sets(2 * half)
+    srcs = [torch.empty(half, dtype=torch.uint8, device=dev).random_(generator=gen) for _ in range(nsets)]
+    dsts = [torch.empty(half, dtype=torch.uint8, device=dev) for _ in range(nsets)]
+    torch.cuda.synchronize()
+    cold = med(lambda: loops.mgpuProbeCopy(ptrs(srcs), ptrs(dsts), nsets, ctypes.c_size_t(half), 100, 10, sp))
+    warm = med(lambda: loops.mgpuProbeCopy(ptrs(srcs[:1]), ptrs(dsts[:1]), 1, ctypes.c_size_t(half), 100, 10, sp))
+    if cold and warm:
+        res["copy_at_headline_size"] = {
+            "bytes": 2 * half, "us_per_launch": round(cold * 10, 3), "GB/s": round(2 * half * 100 / cold / 1e6, 1),
+            "cache_resident_us_per_launch": round(warm * 10, 3),
+            "what": "the same copy kernel at the headline's byte count (12.6 MB in, 12.6 MB out, 3072 blocks): the time "
+                    "a launch of that size costs a kernel that does nothing but move the bytes"}
+    del srcs, dsts
+    sink = torch.zeros(16, device=dev)
+    stamps = torch.zeros(2 * 4096, dtype=torch.int64, device=dev)
+    khz = int(loops.mgpuProbeWallClockKHz())
+    iters = 4096
+    runs = []
+    for waves_per_simd in (1, 2, 3, 4):
+        blocks = 256 * waves_per_simd
+        best = None
+        for _ in range(max(3, repeats // 2)):
+            sc, cc = ctypes.c_uint64(0), ctypes.c_uint64(0)
+            ms = loops.mgpuProbeMfma(ctypes.c_void_p(sink.data_ptr()), ctypes.c_void_p(stamps.data_ptr()), blocks, iters,
+                                     ctypes.byref(sc), ctypes.byref(cc), sp)
+            if ms > 0 and (best is None or ms < best[0]):
+                best = (ms, sc.value, cc.value)
+        if best:
+            ms, sc, cc = best
+            flop = blocks * 4.0 * iters * 4 * 32 * 32 * 16 * 2
+            ghz = sc / cc * khz / 1e6 if cc and khz else None
+            runs.append({"wavefronts_per_simd": waves_per_simd, "TFLOP/s": round(flop / ms / 1e9, 1),
+                         "shader_clock_ghz_in_kernel": ghz and round(ghz, 3),
+                         "clocks_per_mfma": round(sc / (iters * 4.0 * waves_per_simd), 2)})
+    if runs:
+        res["mfma_f16_loop"] = {"runs": runs, "best_TFLOP/s": max(r["TFLOP/s"] for r in runs),
+                                "what": "v_mfma_f32_32x32x16_f16 on four independent accumulators from registers, "
+                                        "4096 x 4 per wavefront, every SIMD of the device; shader clock from clock64() "
+                                        "against the constant-rate wall_clock64()"}
+    return res
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -192,18 +368,22 @@ def main():
         # the launch stream (lib/libmgpu_bench_loops.so): the call rate of a
         # compiled model, which a Python caller cannot reach
         loops = ctypes.CDLL(os.path.join(pkg.LIB_DIR, "libmgpu_bench_loops.so"))
-        for fn in ("mgpuBenchLayerNormF32", "mgpuBenchLayerNormF16", "mgpuBenchAddF32", "mgpuBenchFusedMHAF16"):
+        for fn in ("mgpuBenchLayerNormF32", "mgpuBenchLayerNormF16", "mgpuBenchAddF32", "mgpuBenchFusedMHAF16",
+                   "mgpuBenchBertEncoderLayerF16", "mgpuProbeCopy", "mgpuProbeMfma"):
             getattr(loops, fn).restype = ctypes.c_float
     bench_stream = torch.cuda.Stream()
 
     def ptrs(tensors):
         return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
 
-    def loop_ms(ms):
-        if ms < 0:
+    K, W, R = args.steps, args.warmup, max(1, args.repeats)
+
+    def loop_ms(call):
+        """Median over R timed regions; call() runs one region of a C++ launch loop and returns its milliseconds."""
+        times = [call() for _ in range(R)]
+        if min(times) < 0:
             raise RuntimeError("timed launch loop failed")
-        return ms
-    K, W = args.steps, args.warmup
+        return float(np.median(times))
     only = set(filter(None, args.only.split(",")))
 
     def want(name):
@@ -246,15 +426,14 @@ def main():
         torch.cuda.synchronize()
         sp = ctypes.c_void_p(bench_stream.cuda_stream)
         ln_args = (ctypes.c_void_p(gamma.data_ptr()), ctypes.c_void_p(beta.data_ptr()), ctypes.c_float(1e-5), m, n)
-        ms_cold = loop_ms(loops.mgpuBenchLayerNormF32(ptrs(xs), ptrs(ys), nsets, *ln_args, K, W, sp))
-        ms_warm = loop_ms(loops.mgpuBenchLayerNormF32(ptrs(xs[:1]), ptrs(ys[:1]), 1, *ln_args, K, W, sp))
+        ms_cold = loop_ms(lambda: loops.mgpuBenchLayerNormF32(ptrs(xs), ptrs(ys), nsets, *ln_args, K, W, sp))
+        ms_warm = loop_ms(lambda: loops.mgpuBenchLayerNormF32(ptrs(xs[:1]), ptrs(ys[:1]), 1, *ln_args, K, W, sp))
     else:
-        ms_cold = timer.run(ln32, K, W)
-        ms_warm = timer.run(lambda i: ln32(0), K, W)
+        ms_cold = timer.run(ln32, K, W, R)
+        ms_warm = timer.run(lambda i: ln32(0), K, W, R)
     check()
     headline = hbm_entry("layernorm_f32", "LayerNorm fp32 (32,128,768) eps=1e-5 [configs[1]]", "f32",
                          ln_bytes, ms_cold, K, ms_warm)
-    headline["roofline"]["traffic"] = LN_F32_TRAFFIC_BYTES
     del xs, ys
 
     # ---------------- LayerNorm fp16 ------------------------------------------
@@ -272,11 +451,11 @@ def main():
         if loops:
             torch.cuda.synchronize()
             a16 = (ctypes.c_void_p(gh.data_ptr()), ctypes.c_void_p(bh.data_ptr()), ctypes.c_float(1e-5), m, n)
-            ms = loop_ms(loops.mgpuBenchLayerNormF16(ptrs(xh), ptrs(yh), nsets, *a16, K, W, sp))
-            msw = loop_ms(loops.mgpuBenchLayerNormF16(ptrs(xh[:1]), ptrs(yh[:1]), 1, *a16, K, W, sp))
+            ms = loop_ms(lambda: loops.mgpuBenchLayerNormF16(ptrs(xh), ptrs(yh), nsets, *a16, K, W, sp))
+            msw = loop_ms(lambda: loops.mgpuBenchLayerNormF16(ptrs(xh[:1]), ptrs(yh[:1]), 1, *a16, K, W, sp))
         else:
-            ms = timer.run(ln16, K, W)
-            msw = timer.run(lambda i: ln16(0), K, W)
+            ms = timer.run(ln16, K, W, R)
+            msw = timer.run(lambda i: ln16(0), K, W, R)
         check()
         kernels.append(hbm_entry("layernorm_f16", "LayerNorm fp16 (32,128,768)", "f16",
                                  2 * m * n * 2 + 2 * n * 2, ms, K, msw))
@@ -297,11 +476,11 @@ def main():
 
         if loops:
             torch.cuda.synchronize()
-            ms = loop_ms(loops.mgpuBenchAddF32(ptrs(aa), ptrs(bb), ptrs(cc), nsets, ctypes.c_int64(ne), K, W, sp))
-            msw = loop_ms(loops.mgpuBenchAddF32(ptrs(aa[:1]), ptrs(bb[:1]), ptrs(cc[:1]), 1, ctypes.c_int64(ne), K, W, sp))
+            ms = loop_ms(lambda: loops.mgpuBenchAddF32(ptrs(aa), ptrs(bb), ptrs(cc), nsets, ctypes.c_int64(ne), K, W, sp))
+            msw = loop_ms(lambda: loops.mgpuBenchAddF32(ptrs(aa[:1]), ptrs(bb[:1]), ptrs(cc[:1]), 1, ctypes.c_int64(ne), K, W, sp))
         else:
-            ms = timer.run(add, K, W)
-            msw = timer.run(lambda i: add(0), K, W)
+            ms = timer.run(add, K, W, R)
+            msw = timer.run(lambda i: add(0), K, W, R)
         check()
         kernels.append(hbm_entry("add_f32", "add fp32 (3,640,640) [configs[0]]", "f32", 3 * ne * 4, ms, K, msw))
         del aa, bb, cc
@@ -314,7 +493,7 @@ def main():
         xl = torch.randn((mL, n), device=dev, generator=gen)
         yl = torch.empty_like(xl)
         torch.cuda.synchronize()
-        ms = loop_ms(loops.mgpuBenchLayerNormF32(ptrs([xl]), ptrs([yl]), 1, *ln_args[:3], mL, n, 20, 3, sp))
+        ms = loop_ms(lambda: loops.mgpuBenchLayerNormF32(ptrs([xl]), ptrs([yl]), 1, *ln_args[:3], mL, n, 20, 3, sp))
         check()
         kernels.append(hbm_entry("layernorm_f32_large", f"LayerNorm fp32 ({mL},{n})", "f32",
                                  2 * mL * n * 4 + 2 * n * 4, ms, 20))
@@ -328,8 +507,8 @@ def main():
         gw = 1 + 0.02 * torch.randn(nW, device=dev, generator=gen)
         bw = 0.02 * torch.randn(nW, device=dev, generator=gen)
         torch.cuda.synchronize()
-        ms = loop_ms(loops.mgpuBenchLayerNormF32(ptrs(xw), ptrs(yw), nsW, ctypes.c_void_p(gw.data_ptr()),
-                                                 ctypes.c_void_p(bw.data_ptr()), ctypes.c_float(1e-5), mW, nW, 50, 5, sp))
+        ms = loop_ms(lambda: loops.mgpuBenchLayerNormF32(ptrs(xw), ptrs(yw), nsW, ctypes.c_void_p(gw.data_ptr()),
+                                                         ctypes.c_void_p(bw.data_ptr()), ctypes.c_float(1e-5), mW, nW, 50, 5, sp))
         check()
         kernels.append(hbm_entry("layernorm_f32_wide", f"LayerNorm fp32 ({mW},{nW})", "f32",
                                  2 * mW * nW * 4 + 2 * nW * 4, ms, 50))
@@ -339,7 +518,7 @@ def main():
         al, bl = torch.rand(nl, device=dev, generator=gen), torch.rand(nl, device=dev, generator=gen)
         cl = torch.empty_like(al)
         torch.cuda.synchronize()
-        ms = loop_ms(loops.mgpuBenchAddF32(ptrs([al]), ptrs([bl]), ptrs([cl]), 1, ctypes.c_int64(nl), 20, 3, sp))
+        ms = loop_ms(lambda: loops.mgpuBenchAddF32(ptrs([al]), ptrs([bl]), ptrs([cl]), 1, ctypes.c_int64(nl), 20, 3, sp))
         check()
         kernels.append(hbm_entry("add_f32_large", f"add fp32 ({nl} elements)", "f32", 3 * nl * 4, ms, 20))
         del al, bl, cl
@@ -367,11 +546,11 @@ def main():
         steps = max(20, K // 4)
         if loops:
             torch.cuda.synchronize()
-            ms = loop_ms(loops.mgpuBenchFusedMHAF16(
+            ms = loop_ms(lambda: loops.mgpuBenchFusedMHAF16(
                 ptrs([qkv]), ptrs([out]), 1, ctypes.c_void_p(lens.data_ptr() if lens is not None else None),
                 B, S, H, D, ctypes.c_float(D ** -0.5), int(causal), steps, max(3, W // 4), sp))
         else:
-            ms = timer.run(run, steps, max(3, W // 4))
+            ms = timer.run(run, steps, max(3, W // 4), R)
         check()
         us = ms * 1e3 / steps
         tf = flop_valid / us / 1e6
@@ -425,7 +604,7 @@ def main():
             run(0)                       # first use of the shape: the selection runs here, untimed
             torch.cuda.synchronize()
             steps = max(20, K // 4)
-            ms = Timer(torch, use_graph=True).run(run, steps, 3)
+            ms = Timer(torch, use_graph=True).run(run, steps, 3, R)
             check()
             return ms * 1e3 / steps
 
@@ -467,12 +646,24 @@ def main():
                                         B, S, d, ffn, H, 1e-5, s)
 
         steps = max(10, K // 10)
-        ms = Timer(torch, use_graph=False).run(layer, steps, 3)
+        us_no_alloc = None
+        if loops:
+            # the calls come from a C++ loop, like a compiled model's: seven kernels per call
+            layer(0)  # first use of the GEMM shapes, untimed
+            torch.cuda.synchronize()
+            largs = (ctypes.c_void_p(x.data_ptr()), ptrs(P), None, ctypes.c_void_p(out.data_ptr()),
+                     ctypes.c_int64(B), ctypes.c_int64(S), ctypes.c_int64(d), ctypes.c_int64(ffn), ctypes.c_int64(H),
+                     ctypes.c_float(1e-5))
+            ms = loop_ms(lambda: loops.mgpuBenchBertEncoderLayerF16(*largs, 0, steps, 3, sp))
+            us_no_alloc = loop_ms(lambda: loops.mgpuBenchBertEncoderLayerF16(*largs, 1, steps, 3, sp)) * 1e3 / steps
+        else:
+            ms = Timer(torch, use_graph=False).run(layer, steps, 3, R)
         check()
         us = ms * 1e3 / steps
         flop = 2.0 * B * S * d * (3 * d + d + ffn + ffn) + 4.0 * B * H * S * S * 64
         kernels.append({"name": "bert_layer", "workload": "BERT-base encoder layer fp16 (32,128,768) [configs[4]]",
                         "dtype": "f16", "metric": "us", "value": round(us, 1), "higher_is_better": False,
+                        "us_per_call_no_alloc_entry_point": us_no_alloc and round(us_no_alloc, 1),
                         "roofline": {"bound": "mfma", "achieved": round(flop / us / 1e6, 1),
                                      "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                      "frac": round(flop / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
@@ -495,7 +686,7 @@ def main():
                                             True, True, True, torch.cuda.current_stream().cuda_stream)
 
         steps = max(10, K // 10)
-        ms = Timer(torch, use_graph=False).run(dec, steps, 3)
+        ms = Timer(torch, use_graph=False).run(dec, steps, 3, R)
         check()
         us = ms * 1e3 / steps
         flop = 2.0 * B * S * d * (3 * d + d + 2 * ffn) + 4.0 * B * H * (d // H) * (S * (S + 1) / 2)
@@ -521,7 +712,7 @@ def main():
                            H_, W_, 1, 1, 1, 1, 1, 1, 1, 1, False, False, torch.cuda.current_stream().cuda_stream)
 
         steps = max(10, K // 10)
-        ms = Timer(torch, use_graph=False).run(conv, steps, 3)
+        ms = Timer(torch, use_graph=False).run(conv, steps, 3, R)
         check()
         us = ms * 1e3 / steps
         nbytes = (xc.numel() + wc.numel() + bc.numel() + yc.numel()) * 4
@@ -532,24 +723,20 @@ def main():
                                      "unit": "GB/s", "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None},
                         "algorithmic_bytes": nbytes, "algorithmic_flop": flop})
 
-    # ---------------- CPU baseline: the oracle on the host cores ---------------
+    # ---------------- ceilings measured in this run ------------------------------
+    ceilings = None
+    if loops and not args.no_ceilings:
+        ceilings = measure_ceilings(torch, loops, dev, gen, sp, ptrs, R)
+
+    # ---------------- CPU baseline: the CPU op library on the host cores --------
     cpu = None
     if not args.no_cpu:
-        oracle = ge.load_oracle()
-        rng = np.random.default_rng(20241)
-        x = rng.standard_normal((m, n)).astype(np.float32)
-        g = (1 + 0.02 * rng.standard_normal(n)).astype(np.float32)
-        b = (0.02 * rng.standard_normal(n)).astype(np.float32)
-        threads = oracle.num_threads()
-        oracle.layernorm(x, g, b)
-        reps, t0 = 0, time.perf_counter()
-        while reps < 2000 and time.perf_counter() - t0 < 10.0:
-            oracle.layernorm(x, g, b)
-            reps += 1
-        dt = (time.perf_counter() - t0) / reps
-        cpu = {"value": round(ln_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-               "sample": f"{reps} passes of LayerNorm fp32 (32,128,768) through oracle_layernorm "
-                         f"(fp64 arithmetic, OpenMP, {threads} threads), {dt * 1e6:.0f} us per pass"}
+        cpu_all = cpu_baselines(pkg, m, n, ln_bytes)
+        cpu = cpu_all.pop("layernorm_f32")
+        for e in kernels:
+            key = {"add_f32": "add_f32", "fmha_b32_s128": "fmha_b32_s128", "bert_layer": "bert_layer"}.get(e["name"])
+            if key and key in cpu_all:
+                e["cpu_baseline"] = cpu_all[key]
 
     result = {
         "metric": "LayerNorm GB/s (fp32 (32,128,768)); fMHA TFLOP/s and BERT-base layer us under 'kernels'",
@@ -560,8 +747,9 @@ def main():
                    "launch_mode": ("C++ loop of K calls of the C-ABI entry point" if loops else
                                    "direct ctypes launches" if args.no_graph else "hipGraph of K ctypes launches"),
                    "buffer_sets": rotating_sets(2 * m * n * 4)},
-        "roofline": headline["roofline"], "cache_resident": headline.get("cache_resident"),
-        "cpu_baseline": cpu, "kernels": kernels,
+        "repeats": R, "roofline": headline["roofline"], "cache_resident": headline.get("cache_resident"),
+        "traffic_counted_at_commit": TRAFFIC_COMMIT,
+        "cpu_baseline": cpu, "ceilings": ceilings, "kernels": kernels,
         "device": torch.cuda.get_device_name(0),
         "device_info": device_info(torch),
     }

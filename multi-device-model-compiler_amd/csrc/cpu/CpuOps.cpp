@@ -68,6 +68,17 @@ inline uint16_t floatToHalf(float f) {
 
 extern "C" {
 
+// Thread count of the OpenMP loops below (the CPU baseline is timed at one
+// thread and at all cores).
+void mcpuSetNumThreads(int32_t n) {
+#ifdef _OPENMP
+  if (n > 0) omp_set_num_threads(n);
+#else
+  (void)n;
+#endif
+}
+int32_t mcpuGetNumThreads(void) { return cpuOpsNumThreads(); }
+
 void mcpuMatmul(float *input, float *weight, float *bias, float *output, int64_t M, int64_t N,
                 int64_t K) {
 #pragma omp parallel for schedule(static)

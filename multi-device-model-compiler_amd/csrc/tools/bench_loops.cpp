@@ -64,4 +64,16 @@ float mgpuBenchFusedMHAF16(void *const *qkv, void *const *out, int nsets, const 
       steps, warmup, static_cast<hipStream_t>(stream));
 }
 
+float mgpuBenchBertEncoderLayerF16(const void *x, void *const *params, const int32_t *seqlens, void *out, int64_t B,
+                                   int64_t S, int64_t d, int64_t ffn, int64_t H, float eps, int noAlloc, int steps,
+                                   int warmup, void *stream) {
+  auto *fn = noAlloc ? mgpuBertEncoderLayerF16NoAlloc : mgpuBertEncoderLayerF16;
+  return timed(
+      [&](int) {
+        fn(x, params[0], params[1], params[2], params[3], params[4], params[5], params[6], params[7], params[8],
+           params[9], params[10], params[11], seqlens, out, B, S, d, ffn, H, eps, stream);
+      },
+      steps, warmup, static_cast<hipStream_t>(stream));
+}
+
 } // extern "C"

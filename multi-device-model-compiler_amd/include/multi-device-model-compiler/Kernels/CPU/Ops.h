@@ -14,6 +14,8 @@ bool getOpsFastFlag();                      // :14
 int cpuOpsNumThreads();
 
 extern "C" {
+void mcpuSetNumThreads(int32_t n);
+int32_t mcpuGetNumThreads(void);
 // reference Ops.h:20-22
 void mcpuMatmul(float *input, float *weight, float *bias, float *output, int64_t M, int64_t N,
                 int64_t K);

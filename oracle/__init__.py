@@ -259,6 +259,36 @@ def ref_add_3x640x640(a, b):
     return res
 
 
+def ref_add_seconds(a, b, reruns: int):
+    """Seconds of each of `reruns` runs of the reference's compiled add model
+    (after one untimed run), the model's malloc of its output included and the
+    free of it excluded: what the reference's CPU runner puts its clock around."""
+    import time
+    a, b = _c(a, np.float32), _c(b, np.float32)
+    assert a.shape == (3, 640, 640) and b.shape == (3, 640, 640)
+    ref = ctypes.CDLL(_REF_ADD_PATH)
+    libc = ctypes.CDLL(None)
+    libc.free.argtypes = [ctypes.c_void_p]
+    descs = []
+    for arr in (a, b):
+        d = _MemRef3()
+        d.allocated = d.aligned = arr.ctypes.data
+        d.offset = 0
+        d.sizes[:] = [3, 640, 640]
+        d.strides[:] = [409600, 640, 1]
+        descs.append(d)
+    out = _MemRef3()
+    times = []
+    for i in range(reruns + 1):
+        t0 = time.perf_counter()
+        ref._mlir_ciface_main_graph(ctypes.byref(out), ctypes.byref(descs[0]), ctypes.byref(descs[1]))
+        dt = time.perf_counter() - t0
+        libc.free(out.allocated)
+        if i:
+            times.append(dt)
+    return times
+
+
 def _out_size(size, k, pl, pr, s, d=1):
     return (size + pl + pr - d * (k - 1) - 1) // s + 1
 
