@@ -78,6 +78,9 @@ def parse_args():
     ap.add_argument("--repeats", type=int, default=7, help="timed regions of --steps launches each; the median is reported")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the copy / launch-floor / MFMA-loop probes")
+    ap.add_argument("--fmha-phases", action="store_true",
+                    help="also run the attention kernel's profiling entry point at b32 s512 h12 d64 and report where a "
+                         "block's time goes (prologue, tiles, epilogue) from the kernel's own clocks")
     ap.add_argument("--graph", action="store_true",
                     help="time a hipGraph of K ctypes launches instead of the C++ launch loops")
     ap.add_argument("--no-graph", action="store_true", help="with --graph: enqueue the ctypes launches directly")
@@ -281,6 +284,55 @@ def cpu_baselines(pkg, m, n, ln_bytes) -> dict:
                                                                   i64(ffn), i64(H), ctypes.c_float(1e-5)),
                              4.0, 10, lambda s: s * 1e6, "us", "BERT-base encoder layer fp16 (32,128,768)")
     return out
+
+
+def fmha_phases(torch, lib, loops, dev, gen, B=32, S=512, H=12) -> dict:
+    """Per-block clock stamps of the attention kernel (mgpuFusedMHAF16Profile):
+    how long a block spends before its first tile, per tile, and after its last
+    tile, and how the blocks fill the launch."""
+    D = 64
+    qkv = (torch.randn((B, S, 3, H, D), device=dev, generator=gen) / 8).half()
+    out = torch.empty((B, S, H * D), device=dev, dtype=torch.float16)
+    nblocks = B * H * ((S + 127) // 128)
+    stamps = torch.zeros(nblocks * 10, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(3):
+        got = lib.mgpuFusedMHAF16Profile(qkv.data_ptr(), out.data_ptr(), B, S, H, D ** -0.5, stamps.data_ptr(), stream)
+    torch.cuda.synchronize()
+    if got != nblocks:
+        raise RuntimeError("mgpuFusedMHAF16Profile failed")
+    t = stamps.cpu().numpy().reshape(nblocks, 10).astype(np.float64)
+    khz = int(loops.mgpuProbeWallClockKHz()) if loops else 100000
+    wall_us = lambda ticks: ticks / khz * 1e3
+    k0 = t[:, 4].min()
+    start_us, end_us = wall_us(t[:, 4] - k0), wall_us(t[:, 5] - k0)
+    total_us = end_us.max()
+    ghz = float(np.median((t[:, 3] - t[:, 0]) / np.maximum(1.0, (t[:, 5] - t[:, 4])) * khz / 1e6))
+    tiles = (S + 63) // 64
+    pro, loop, epi = t[:, 1] - t[:, 0], t[:, 2] - t[:, 1], t[:, 3] - t[:, 2]
+    first = start_us < 1.0  # blocks resident from the start of the launch
+    q = lambda a: [round(float(np.percentile(a, p)), 1) for p in (10, 50, 90)]
+    return {
+        "shape": f"b{B} s{S} h{H} d{D}", "blocks": nblocks, "tiles_per_block": tiles,
+        "kernel_us_first_entry_to_last_exit": round(float(total_us), 2),
+        "shader_clock_ghz": round(ghz, 3),
+        "blocks_resident_at_start": int(first.sum()),
+        "last_block_entry_us": round(float(start_us.max()), 2),
+        "cycles_p10_p50_p90": {
+            "prologue_entry_to_first_tile": q(pro), "prologue_of_blocks_resident_at_start": q(pro[first]),
+            "prologue_of_later_blocks": q(pro[~first]) if (~first).any() else None,
+            "loop_per_tile": q(loop / tiles), "epilogue_last_tile_to_stores_issued": q(epi),
+            "per_tile_wait_for_tile_and_barrier": q(t[:, 6] / tiles), "per_tile_score_mfmas": q(t[:, 7] / tiles),
+            "per_tile_softmax": q(t[:, 8] / tiles), "per_tile_pv_mfmas": q(t[:, 9] / tiles)},
+        "share_of_block_lifetime": {
+            "prologue": round(float(pro.sum() / (pro + loop + epi).sum()), 3),
+            "tiles": round(float(loop.sum() / (pro + loop + epi).sum()), 3),
+            "epilogue": round(float(epi.sum() / (pro + loop + epi).sum()), 3)},
+        "block_lifetime_us_p50": round(float(np.median(end_us - start_us)), 2),
+        "mfma_cycles_per_tile_per_simd": 3 * 16 * 32,
+        "note": "loop_per_tile is one wavefront's time per 64-key tile with 3 wavefronts sharing the SIMD: the SIMD's "
+                "matrix pipe needs 3 x 16 x 32 = 1536 cycles for the three tiles that pass in that time",
+    }
 
 
 def measure_ceilings(torch, loops, dev, gen, sp, ptrs, repeats) -> dict:
@@ -728,6 +780,8 @@ def main():
     if loops and not args.no_ceilings:
         ceilings = measure_ceilings(torch, loops, dev, gen, sp, ptrs, R)
 
+    phases = fmha_phases(torch, lib, loops, dev, gen) if args.fmha_phases else None
+
     # ---------------- CPU baseline: the CPU op library on the host cores --------
     cpu = None
     if not args.no_cpu:
@@ -749,7 +803,7 @@ def main():
                    "buffer_sets": rotating_sets(2 * m * n * 4)},
         "repeats": R, "roofline": headline["roofline"], "cache_resident": headline.get("cache_resident"),
         "traffic_counted_at_commit": TRAFFIC_COMMIT,
-        "cpu_baseline": cpu, "ceilings": ceilings, "kernels": kernels,
+        "cpu_baseline": cpu, "ceilings": ceilings, "fmha_phases": phases, "kernels": kernels,
         "device": torch.cuda.get_device_name(0),
         "device_info": device_info(torch),
     }

@@ -121,6 +121,18 @@ void mgpuFusedMHABF16CuSeqlens(const void *qkv, const int32_t *cu_seqlens, void 
                                int32_t max_s, int32_t H, int32_t D, float scale, int32_t causal,
                                mgpuStream_t stream);
 
+/* Profiling aid, no counterpart in the reference: mgpuFusedMHAF16 for head_dim
+ * 64 without masks, with the kernel's own clocks recorded per 256-thread block.
+ * stamps receives ten uint64 per block (device memory, 10 * return value
+ * entries; blocks = B * H * ceil(S / 128)), all from wavefront 0 of the block:
+ * the shader clock at block entry, when the first K/V tile has landed, after
+ * the last tile, after the output stores were issued; the device-wide
+ * constant-rate clock at entry and exit; and the shader clocks, summed over the
+ * block's tiles, spent waiting for a tile to land, in the score MFMAs, in the
+ * softmax and in the P.V MFMAs.  Returns the number of blocks (0 on error). */
+int64_t mgpuFusedMHAF16Profile(const void *qkv, void *out, int32_t B, int32_t S, int32_t H, float scale,
+                               uint64_t *stamps, mgpuStream_t stream);
+
 /* ---- casts (Utils.h:6-8; lib/Kernels/GPU/Utils.cu:85-103) ------------- */
 void mgpuCastF32ToF16(void *dst, const float *src, size_t size, mgpuStream_t stream);
 void mgpuCastF16ToF32(float *dst, const void *src, size_t size, mgpuStream_t stream);

@@ -59,6 +59,7 @@ OPS_SIGNATURES = {
     "mgpuFusedMHABF16": (None, [_c_void_p] * 3 + [_c_int32] * 4 + [_c_float, _c_int32, _c_void_p]),
     "mgpuFusedMHAF16CuSeqlens": (None, [_c_void_p] * 3 + [_c_int32] * 4 + [_c_float, _c_int32, _c_void_p]),
     "mgpuFusedMHABF16CuSeqlens": (None, [_c_void_p] * 3 + [_c_int32] * 4 + [_c_float, _c_int32, _c_void_p]),
+    "mgpuFusedMHAF16Profile": (_c_int64, [_c_void_p, _c_void_p] + [_c_int32] * 3 + [_c_float, _c_void_p, _c_void_p]),
     "mgpuCastF32ToF16": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
     "mgpuCastF16ToF32": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
     "mgpuCastF32ToBF16": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),

@@ -33,6 +33,7 @@ template <typename F> void guarded(F &&f) noexcept {
 }
 
 inline hipStream_t S(mgpuStream_t s) { return reinterpret_cast<hipStream_t>(s); }
+inline hipStream_t S_(mgpuStream_t s) { return reinterpret_cast<hipStream_t>(s); } // where a parameter is called S
 
 } // namespace
 
@@ -231,6 +232,13 @@ void mgpuFusedMHABF16CuSeqlens(const void *qkv, const int32_t *cu_seqlens, void 
   guarded([&] {
     mgpu::fusedMHACuSeqlens(mgpu::DType::BF16, qkv, cu_seqlens, out, B, max_s, H, D, scale, causal != 0, S(stream));
   });
+}
+
+int64_t mgpuFusedMHAF16Profile(const void *qkv, void *out, int32_t B, int32_t S, int32_t H, float scale,
+                               uint64_t *stamps, mgpuStream_t stream) {
+  int64_t blocks = 0;
+  guarded([&] { blocks = mgpu::fusedMHAProfile(qkv, out, B, S, H, scale, stamps, S_(stream)); });
+  return blocks;
 }
 
 void mgpuCastF32ToF16(void *dst, const float *src, size_t size, mgpuStream_t stream) {

@@ -108,12 +108,25 @@ template <int D> struct Geo {
 constexpr float kSumLimit = 32768.0f;
 constexpr float kSumFloor = 0.015625f;
 
-template <typename T, int D, int NQ, bool CAUSAL>
+// TRACE (the profiling entry point only): wavefront 0 of every block records
+// the shader clock at entry, when its first tile has landed, after its last
+// tile and after its stores, the device-wide constant clock at entry and
+// exit, and the shader clocks its tiles spent waiting for the tile to land
+// (wait + barrier), in the score MFMAs, in the softmax and in the P.V MFMAs:
+// ten uint64 per block in `stamps`.
+template <typename T, int D, int NQ, bool CAUSAL, bool TRACE = false>
 __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_kernel(const uint16_t *__restrict__ qkv,
                                                               const int32_t *__restrict__ seqlens,
                                                               const int32_t *__restrict__ cuSeqlens,
                                                               uint16_t *__restrict__ out, int S, int H,
-                                                              int nQB, float scale_log2e, int pairItems) {
+                                                              int nQB, float scale_log2e, int pairItems,
+                                                              uint64_t *__restrict__ stamps) {
+  uint64_t tEntry = 0, wEntry = 0, tFirstTile = 0, tLoopEnd = 0;
+  uint64_t cWait = 0, cScores = 0, cSoftmax = 0, cPV = 0, tMark = 0;
+  if (TRACE) {
+    tEntry = clock64();
+    wEntry = wall_clock64();
+  }
   using M = Mma<T>;
   using v8 = typename M::v8;
   using v4 = typename M::v4;
@@ -288,12 +301,14 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   }
 
   for (int kt = 0; kt < nkt; kt++) {
+    if (TRACE) tMark = clock64();
     // The loads of tile kt (and of nothing later) must have landed; the barrier
     // makes every wavefront's share visible and also says that everybody is
     // done with tile kt-1, whose stage the next load may overwrite.
     if (kt + 1 < nkt) asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); // vmcnt(4): tile kt+1 may still fly
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");              // vmcnt(0)
     __syncthreads();
+    if (TRACE && kt == 0) tFirstTile = clock64();
     if (kt + kStages - 1 < nkt) issueTile(kt + kStages - 1);
 
     const uint32_t stageOff = (uint32_t)((kt % kStages) * (2 * kTileBytes));
@@ -323,6 +338,11 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
 #pragma unroll
     for (int db = 0; db < G::DB; db++) vp[db] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kTileBytes + vfrag[db]);
 
+    if (TRACE) {
+      const uint64_t t = clock64();
+      cWait += t - tMark;
+      tMark = t;
+    }
     // ---- S^T = K Q^T -------------------------------------------------------
     f32x16 accS[NQ][G::KB];
     __builtin_amdgcn_s_setprio(2); // MFMA phases outrank the softmax phases of the SIMD's other wavefronts
@@ -343,6 +363,13 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
     }
 
     __builtin_amdgcn_s_setprio(0);
+    if (TRACE) {
+      // a use of the last accumulator makes the stamp wait for the MFMAs
+      asm volatile("" ::"v"(accS[NQ - 1][G::KB - 1][15]));
+      const uint64_t t = clock64();
+      cScores += t - tMark;
+      tMark = t;
+    }
     const bool needMask = (key0 + kBN > kvlen) || (CAUSAL && key0 + kBN - 1 > q0);
     v8 pf[NQ][G::KB][2];
 #pragma unroll
@@ -403,6 +430,11 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
       l_run[qi] += lsum;
     }
 
+    if (TRACE) {
+      const uint64_t t = clock64();
+      cSoftmax += t - tMark;
+      tMark = t;
+    }
     // ---- O^T += V^T P^T ----------------------------------------------------
     __builtin_amdgcn_s_setprio(2);
 #pragma unroll
@@ -421,8 +453,13 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
       }
     }
     __builtin_amdgcn_s_setprio(0);
+    if (TRACE) {
+      asm volatile("" ::"v"(accO[NQ - 1][G::DB - 1][15]));
+      cPV += clock64() - tMark;
+    }
   }
 
+  if (TRACE) tLoopEnd = clock64();
   // ---- normalise, transpose through LDS, store whole rows ------------------
   __syncthreads(); // every wavefront is done reading the K / V tiles
   constexpr int kOS = G::OS;
@@ -461,6 +498,20 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   // the next part's tiles land in the ring the staging area sits in
   if (part + 1 < nParts) __syncthreads();
   } // part
+  if (TRACE && threadIdx.x == 0) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the output stores have left the wavefront
+    uint64_t *rec = stamps + (size_t)blockIdx.x * 10;
+    rec[0] = tEntry;
+    rec[1] = tFirstTile;
+    rec[2] = tLoopEnd;
+    rec[3] = clock64();
+    rec[4] = wEntry;
+    rec[5] = wall_clock64();
+    rec[6] = cWait;
+    rec[7] = cScores;
+    rec[8] = cSoftmax;
+    rec[9] = cPV;
+  }
 }
 
 // Compute units of the current device (asked once per device).
@@ -491,9 +542,9 @@ void launch(const void *qkv, const int32_t *seqlens, const int32_t *cuSeqlens, v
   const auto *in = static_cast<const uint16_t *>(qkv);
   auto *o = static_cast<uint16_t *>(out);
   if (causal)
-    fmha_fwd_kernel<T, D, NQ, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0);
+    fmha_fwd_kernel<T, D, NQ, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, nullptr);
   else
-    fmha_fwd_kernel<T, D, NQ, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0);
+    fmha_fwd_kernel<T, D, NQ, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, nullptr);
   MGPU_CHECK_LAUNCH("fmha_fwd_kernel");
 }
 
@@ -527,6 +578,22 @@ void fusedMHAChecked(DType dt, const void *qkv, const int32_t *seqlens, const in
 void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int B, int S, int H,
               int D, float scale, bool causal, hipStream_t stream) {
   fusedMHAChecked(dt, qkv, seqlens, nullptr, out, B, S, H, D, scale, causal, stream);
+}
+
+// mgpuFusedMHAF16Profile: the fp16, head_dim 64, unmasked kernel with TRACE on.
+int64_t fusedMHAProfile(const void *qkv, void *out, int B, int S, int H, float scale, uint64_t *stamps,
+                        hipStream_t stream) {
+  if (B <= 0 || S <= 0 || H <= 0) fail("fusedMHAProfile: empty shape");
+  if (!qkv || !out || !stamps) fail("fusedMHAProfile: null pointer");
+  if (!aligned16(qkv) || !aligned16(out)) fail("fusedMHAProfile: qkv and out must be 16-byte aligned");
+  const int nQB = (S + 127) / 128;
+  const int64_t blocks = (int64_t)B * H * nQB;
+  if (blocks > 0x7fffffffLL) fail("fusedMHAProfile: problem too large for one launch");
+  fmha_fwd_kernel<_Float16, 64, 1, false, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+      static_cast<const uint16_t *>(qkv), nullptr, nullptr, static_cast<uint16_t *>(out), S, H, nQB,
+      scale * 1.44269504088896340736f, 0, stamps);
+  MGPU_CHECK_LAUNCH("fmha_fwd_kernel (profile)");
+  return blocks;
 }
 
 void fusedMHACuSeqlens(DType dt, const void *qkv, const int32_t *cuSeqlens, void *out, int B, int maxS, int H,

@@ -34,6 +34,13 @@ void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int 
 void fusedMHACuSeqlens(DType dt, const void *qkv, const int32_t *cuSeqlens, void *out, int B, int maxS, int H,
                        int D, float scale, bool causal, hipStream_t stream);
 
+// The fp16 head_dim-64 unmasked kernel with per-block clock stamps: ten uint64 per
+// block (shader clock at entry, first tile landed, last tile done, stores issued;
+// constant-rate clock at entry and exit; clocks spent waiting for tiles, in the
+// score MFMAs, in the softmax, in the P.V MFMAs).  Returns the number of blocks.
+int64_t fusedMHAProfile(const void *qkv, void *out, int B, int S, int H, float scale, uint64_t *stamps,
+                        hipStream_t stream);
+
 void castF32ToF16(void *dst, const float *src, size_t size, hipStream_t stream);
 void castF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream);
 void castF32ToBF16(void *dst, const float *src, size_t size, hipStream_t stream);
