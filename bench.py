@@ -78,6 +78,9 @@ def parse_args():
     ap.add_argument("--repeats", type=int, default=7, help="timed regions of --steps launches each; the median is reported")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the copy / launch-floor / MFMA-loop probes")
+    ap.add_argument("--tune-gemm", action="store_true",
+                    help="measure the four GEMM shapes of the BERT-base layer with mgpuMatmulExTune (library candidates "
+                         "against the hand-written kernel) and print the lines of csrc/kernels/gemm_table.inc on stderr")
     ap.add_argument("--fmha-phases", action="store_true",
                     help="also run the attention kernel's profiling entry point at b32 s512 h12 d64 and report where a "
                          "block's time goes (prologue, tiles, epilogue) from the kernel's own clocks")
@@ -392,6 +395,20 @@ def measure_ceilings(torch, loops, dev, gen, sp, ptrs, repeats) -> dict:
                                 "what": "v_mfma_f32_32x32x16_f16 on four independent accumulators from registers, "
                                         "4096 x 4 per wavefront, every SIMD of the device; shader clock from clock64() "
                                         "against the constant-rate wall_clock64()"}
+    mix = {}
+    for mode, name in ((0, "interleaved"), (1, "in_phases")):
+        per = {}
+        for waves_per_simd in (1, 2, 3, 4):
+            c = loops.mgpuProbeFmhaMix(ctypes.c_void_p(sink.data_ptr()), ctypes.c_void_p(stamps.data_ptr()),
+                                       256 * waves_per_simd, 400, mode, sp)
+            if c > 0:
+                per[str(waves_per_simd)] = round(c / waves_per_simd, 1)
+        mix[name] = per
+    res["fmha_d64_tile_instruction_mix"] = {
+        "simd_clocks_per_tile_by_wavefronts_per_simd": mix, "mfma_clocks_per_tile": 16 * 32,
+        "what": "the instructions of one 64-key x 32-query tile of the head_dim-64 attention kernel (16 MFMAs, 32 fma / exp2 / "
+                "add, 16 converts, 24 LDS operand reads whose data nobody waits for), no barrier, no tile loads: the clocks a "
+                "SIMD needs per tile for that mix, finely interleaved and in the kernel's three phases"}
     return res
 
 
@@ -423,6 +440,7 @@ def main():
         for fn in ("mgpuBenchLayerNormF32", "mgpuBenchLayerNormF16", "mgpuBenchAddF32", "mgpuBenchFusedMHAF16",
                    "mgpuBenchBertEncoderLayerF16", "mgpuProbeCopy", "mgpuProbeMfma"):
             getattr(loops, fn).restype = ctypes.c_float
+        loops.mgpuProbeFmhaMix.restype = ctypes.c_double
     bench_stream = torch.cuda.Stream()
 
     def ptrs(tensors):
@@ -596,13 +614,14 @@ def main():
                                 out.data_ptr(), B, S, H, D, D ** -0.5, int(causal), s)
 
         steps = max(20, K // 4)
+        warm = max(10, W)  # enough launches for the clocks to settle under matrix load
         if loops:
             torch.cuda.synchronize()
             ms = loop_ms(lambda: loops.mgpuBenchFusedMHAF16(
                 ptrs([qkv]), ptrs([out]), 1, ctypes.c_void_p(lens.data_ptr() if lens is not None else None),
-                B, S, H, D, ctypes.c_float(D ** -0.5), int(causal), steps, max(3, W // 4), sp))
+                B, S, H, D, ctypes.c_float(D ** -0.5), int(causal), steps, warm, sp))
         else:
-            ms = timer.run(run, steps, max(3, W // 4), R)
+            ms = timer.run(run, steps, warm, R)
         check()
         us = ms * 1e3 / steps
         tf = flop_valid / us / 1e6
@@ -640,8 +659,9 @@ def main():
 
     # ---------------- GEMM with fused epilogue ---------------------------------
     # The four GEMMs of the BERT-base layer at 4096 tokens.  mgpuMatmulExF16 runs whichever of the library (+ a
-    # separate GELU pass where there is one) and the hand-written MFMA kernel its first-use measurement kept;
-    # mgpuGemmMfmaF16 is the hand-written kernel by itself.
+    # separate GELU pass where there is one) and the hand-written MFMA kernel the committed table names for the
+    # shape; mgpuGemmMfmaF16 is the hand-written kernel by itself.  With --tune-gemm the shape is first measured
+    # on this device (mgpuMatmulExTune) and the table line that measurement gives is printed.
     def gemm_case(name, workload, M_, K_, N_, act, residual):
         x = torch.randn((M_, K_), device=dev, generator=gen).half()
         wt = (0.02 * torch.randn((K_, N_), device=dev, generator=gen)).half()
@@ -653,18 +673,24 @@ def main():
             def run(i):
                 fn(x.data_ptr(), wt.data_ptr(), bias.data_ptr(), y.data_ptr(), res.data_ptr() if residual else None,
                    M_, N_, K_, 1, act, int(residual), torch.cuda.current_stream().cuda_stream)
-            run(0)                       # first use of the shape: the selection runs here, untimed
+            run(0)                       # first use of the shape (descriptors, code), untimed
             torch.cuda.synchronize()
             steps = max(20, K // 4)
             ms = Timer(torch, use_graph=True).run(run, steps, 3, R)
             check()
             return ms * 1e3 / steps
 
+        tuned = None
+        if args.tune_gemm:
+            tuned = int(lib.mgpuMatmulExTune(1, M_, N_, K_, 1, act, int(residual)))
+            check()
+            print(f"{{1, {M_}, {N_}, {K_}, 1, {act}, {int(residual)}, {tuned}}},", file=sys.stderr)
         us_auto, us_mfma = gemm(lib.mgpuMatmulExF16), gemm(lib.mgpuGemmMfmaF16)
         flop = 2.0 * M_ * N_ * K_
         kernels.append({"name": name, "workload": workload,
                         "dtype": "f16", "metric": "TFLOP/s", "value": round(flop / us_auto / 1e6, 1),
                         "us_per_launch": round(us_auto, 2), "us_per_launch_gemm_mfma": round(us_mfma, 2),
+                        "kernel_kept_by_tuning_in_this_run": tuned if tuned is None else ("gemm_mfma" if tuned else "library"),
                         "roofline": {"bound": "mfma", "achieved": round(flop / us_auto / 1e6, 1),
                                      "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                      "frac": round(flop / us_auto / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},

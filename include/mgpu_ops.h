@@ -185,6 +185,18 @@ void mgpuMatmulExBF16(void *input, void *weight, void *bias, void *output, void 
                       int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
                       int32_t hasResidual, mgpuStream_t stream);
 
+/* mgpuMatmulEx* only enqueue: which kernel serves a shape (the library's or the
+ * hand-written MFMA kernel below) comes from a table decided offline and a
+ * fixed rule.  A caller who wants a shape measured on its own device asks for
+ * it here, once, OUTSIDE any stream capture: the call allocates scratch
+ * operands, times the library's candidates and the hand-written kernel
+ * (synchronous, tens of milliseconds) and keeps the winner for the rest of the
+ * process.  dtype: 0 fp32, 1 fp16, 2 bf16.  Returns 1 when the hand-written
+ * kernel was kept, 0 for the library, -1 on error.  No counterpart in the
+ * reference (it takes cuBLASLt's first heuristic, Ops.cu:186-200). */
+int32_t mgpuMatmulExTune(int32_t dtype, int64_t M, int64_t N, int64_t K, int32_t hasBias,
+                         int32_t hasRelu, int32_t hasResidual);
+
 /* The hand-written MFMA kernel that serves mgpuMatmulExF16 / BF16 where it is
  * the faster path, callable by itself (no counterpart in the reference):
  * same arguments; M a multiple of 128, N of 128 or 96, K of 32, operands
@@ -228,8 +240,8 @@ void mgpuBertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, 
  * live in a fixed 48 MiB device array inside the library (one copy per GPU,
  * held until the process ends) and all four GEMMs run on the hand-written MFMA
  * kernel.  Limits, each an error reported through mgpuOpsTakeLastError():
- *   batch*seq_len * (max(4*d_model, feed_forward_dim) + 3*d_model) * 2 bytes
- *   must fit in 48 MiB (BERT-base (32,128,768), ffn 3072: 42 MiB);
+ *   batch*seq_len * (max(4*d_model, feed_forward_dim) + 2*d_model) * 2 bytes
+ *   must fit in 48 MiB (BERT-base (32,128,768), ffn 3072: 36 MiB);
  *   batch*seq_len a multiple of 128, d_model and feed_forward_dim multiples
  *   of 128 (or 96) and of 32, operands 16-byte aligned.
  * Every call on one GPU shares that GPU's array: calls that overlap in time on

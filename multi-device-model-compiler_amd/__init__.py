@@ -71,6 +71,7 @@ OPS_SIGNATURES = {
     "mgpuPool2d": (None, [_c_void_p] * 2 + [_c_int64] * 15 + [_c_void_p]),
     "mgpuMatmulExF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuMatmulExBF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
+    "mgpuMatmulExTune": (_c_int32, [_c_int32] + [_c_int64] * 3 + [_c_int32] * 3),
     "mgpuGemmMfmaF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuGemmMfmaBF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuMatmulExF32": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),

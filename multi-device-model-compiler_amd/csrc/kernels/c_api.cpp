@@ -328,6 +328,15 @@ void mgpuGemmMfmaBF16(void *input, void *weight, void *bias, void *output, void 
                     S(stream));
   });
 }
+int32_t mgpuMatmulExTune(int32_t dtype, int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
+                         int32_t hasResidual) {
+  int32_t kept = -1;
+  guarded([&] {
+    if (dtype < 0 || dtype > 2) mgpu::fail("mgpuMatmulExTune: dtype is 0 (fp32), 1 (fp16) or 2 (bf16)");
+    kept = mgpu::tuneMatmulEx(static_cast<mgpu::DType>(dtype), M, N, K, hasBias != 0, hasRelu, hasResidual != 0) ? 1 : 0;
+  });
+  return kept;
+}
 void mgpuMatmulExBF16(void *input, void *weight, void *bias, void *output, void *residual,
                       int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
                       int32_t hasResidual, mgpuStream_t stream) {

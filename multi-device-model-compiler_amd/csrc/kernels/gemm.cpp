@@ -8,15 +8,23 @@
 //    descriptors on every call and caches only the heuristic result;
 //  * fp16 / bf16 inputs accumulate in fp32 (HIPBLAS_COMPUTE_32F); the reference
 //    asks for fp16 accumulation (Ops.cu:164-167);
-//  * the algorithm is chosen by measurement: the first use of a shape times the
-//    library's top candidates on scratch operands of that shape and keeps the
-//    fastest (the heuristic's first answer is not always it at M = 4096);
 //  * GELU is applied by an exact-erf kernel after a bias-only epilogue, because
 //    the library's fused GELU is the tanh approximation;
-//  * fp16 / bf16 shapes that the hand-written MFMA kernel (gemm_mfma.hip)
-//    accepts are timed on it as well, GELU pass included on the library's
-//    side, and the faster path is kept for the shape.  MGPU_GEMM_KERNEL=library
-//    or =mfma in the environment overrides the measurement.
+//  * a call only enqueues: which of the two kernels serves a shape - the
+//    library or the hand-written MFMA kernel of gemm_mfma.hip - comes from a
+//    table decided offline (gemm_table.inc, written by `bench.py --tune-gemm`
+//    from measurements on an MI355X) and, for shapes the table does not hold,
+//    from a fixed rule; the library runs the heuristic's first algorithm.
+//    MGPU_GEMM_KERNEL=library or =mfma in the environment overrides both.  A
+//    caller who wants a shape measured on its own device asks for it
+//    explicitly with tuneMatmulEx (mgpuMatmulExTune in the C ABI), outside any
+//    stream capture: that call allocates scratch operands, times the
+//    library's candidates and the hand-written kernel, and keeps the winner
+//    for the rest of the process;
+//  * the library's workspace is per caller stream (allocated on a stream's
+//    first library GEMM outside a capture), so GEMMs on different streams never
+//    share one; a stream first seen under capture gets an algorithm that needs
+//    no workspace.
 #include "common.hpp"
 #include "mgpu_ops_internal.hpp"
 
@@ -35,9 +43,25 @@ namespace mgpu {
 namespace {
 
 hipblasLtHandle_t ltHandle = nullptr;
-void *workspace = nullptr;
 constexpr size_t workspaceSize = 32u * 1024u * 1024u;
 std::mutex planMutex;
+std::map<hipStream_t, void *> workspaceOf; // per caller stream, see the header comment
+
+bool isCapturing(hipStream_t s) {
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  return hipStreamIsCapturing(s, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone;
+}
+
+// The stream's workspace; null when it has none yet and none can be made now (capture).
+void *workspaceFor(hipStream_t s) {
+  auto it = workspaceOf.find(s);
+  if (it != workspaceOf.end()) return it->second;
+  if (isCapturing(s)) return nullptr;
+  void *ws = nullptr;
+  MGPU_CHECK_HIP(hipMalloc(&ws, workspaceSize));
+  workspaceOf[s] = ws;
+  return ws;
+}
 
 void checkBlas(hipblasStatus_t status, const char *where) {
   if (status != HIPBLAS_STATUS_SUCCESS)
@@ -48,9 +72,30 @@ void checkBlas(hipblasStatus_t status, const char *where) {
 struct Plan {
   hipblasLtMatmulDesc_t op = nullptr;
   hipblasLtMatrixLayout_t a = nullptr, b = nullptr, d = nullptr;
-  hipblasLtMatmulAlgo_t algo;
+  hipblasLtMatmulAlgo_t algo;          // the heuristic's first answer (or the tuned one)
+  size_t algoWorkspace = 0;
+  hipblasLtMatmulAlgo_t algoNoWs;      // the first answer that needs no workspace
+  bool hasNoWs = false;
   bool handWritten = false; // serve the shape with gemm_mfma.hip when the operands allow it
 };
+
+// Shapes decided offline: {type (1 fp16, 2 bf16), M, N, K, hasBias, act, hasResidual, hand-written kernel?}.
+struct TableEntry {
+  int dt;
+  int64_t M, N, K;
+  int hasBias, act, hasResidual, handWritten;
+};
+const TableEntry kTable[] = {
+#include "gemm_table.inc"
+};
+
+// Which kernel serves a shape nobody measured: the hand-written one where it can pay -
+// reductions up to 1024 deep, a GELU to fuse, or at most one 128-row tile per CU (its
+// eight-wavefront form).  On long reductions over many tiles the library's steady state
+// is ahead.
+bool ruleSaysHandWritten(int64_t M, int64_t N, int64_t K, int act) {
+  return K <= 1024 || act == ACT_GELU || (M / 128) * (N / 128) <= numComputeUnits();
+}
 
 // 0: measure, 1: always the library, 2: the hand-written kernel wherever it applies
 int forcedKernel() {
@@ -98,12 +143,13 @@ int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *resu
                      int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual,
                      bool *handWritten) {
   const size_t eb = dt == DType::F32 ? 4 : 2;
-  void *in = nullptr, *w = nullptr, *out = nullptr, *bias = nullptr;
+  void *in = nullptr, *w = nullptr, *out = nullptr, *bias = nullptr, *workspace = nullptr;
   hipStream_t s = nullptr;
   hipEvent_t e0 = nullptr, e1 = nullptr;
   int best = 0;
   const bool ready = hipMalloc(&in, (size_t)M * K * eb) == hipSuccess && hipMalloc(&w, (size_t)K * N * eb) == hipSuccess &&
                      hipMalloc(&out, (size_t)M * N * eb) == hipSuccess && hipMalloc(&bias, (size_t)N * eb) == hipSuccess &&
+                     hipMalloc(&workspace, workspaceSize) == hipSuccess &&
                      hipStreamCreate(&s) == hipSuccess && hipEventCreate(&e0) == hipSuccess &&
                      hipEventCreate(&e1) == hipSuccess;
   if (ready) {
@@ -148,14 +194,7 @@ int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *resu
     }
     // The hand-written kernel on the same operands (`out` doubles as the residual).
     const void *biasArg = hasBias ? bias : nullptr, *resArg = hasResidual ? out : nullptr;
-    // Only where it can pay: reductions up to 1024 deep, a GELU to fuse, or at most one
-    // 128-row tile per CU (its eight-wavefront form).  On long reductions over many
-    // tiles the library's steady state (0.9-1.3 PFLOP/s) is ahead of this kernel's
-    // (0.75-1.0), and there the kernel also loses more than the library when another
-    // stream loads the memory system at the same time (the reference layer's weight
-    // casts do), which a burst of launches on an idle device does not show.
-    const bool candidate = K <= 1024 || act == ACT_GELU || (M / 128) * (N / 128) <= numComputeUnits();
-    if (candidate && bestMs >= 0.0f && gemmMfmaSupports(dt, in, w, biasArg, resArg, out, M, N, K)) {
+    if (bestMs >= 0.0f && gemmMfmaSupports(dt, in, w, biasArg, resArg, out, M, N, K)) {
       // Both paths in alternating runs of twenty launches, three runs each, so that
       // they meet the same clocks: a lone burst of a kernel that has the device to
       // itself for a millisecond runs faster than the same kernel in a layer.
@@ -200,18 +239,25 @@ int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *resu
   if (e0) (void)hipEventDestroy(e0);
   if (e1) (void)hipEventDestroy(e1);
   if (s) (void)hipStreamDestroy(s);
-  for (void *ptr : {in, w, out, bias})
+  for (void *ptr : {in, w, out, bias, workspace})
     if (ptr) (void)hipFree(ptr);
   (void)hipGetLastError();
   return best;
 }
 
-const Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act,
-                    bool hasResidual, hipStream_t stream) {
+// Builds (once per shape, flags and type) the library's descriptors and picks its
+// algorithms; decides which kernel serves the shape.  No measurement, no allocation
+// beyond the library's host-side descriptors.  With `tune` the caller has asked for the
+// measurement (tuneMatmulEx).
+Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual, bool tune) {
   const bool relu = act == ACT_RELU;
   const Key key{M, N, K, (int)hasBias, act, (int)hasResidual, (int)dt};
   auto it = plans.find(key);
-  if (it != plans.end()) return it->second;
+  if (it != plans.end() && !tune) return it->second;
+  if (it != plans.end()) {
+    destroyPlan(it->second);
+    plans.erase(it);
+  }
 
   Plan p;
   const hipDataType t = dataType(dt);
@@ -252,10 +298,25 @@ const Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int
          std::to_string(N) + " K=" + std::to_string(K));
   }
   p.algo = results[0].algo;
-  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-  const bool capturing = hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone;
-  if (!capturing) // a capturing caller gets the heuristic's first answer
-    p.algo = results[fastestCandidate(p, results, returned, dt, M, N, K, hasBias, act, hasResidual, &p.handWritten)].algo;
+  p.algoWorkspace = results[0].workspaceSize;
+  for (int c = 0; c < returned && !p.hasNoWs; c++)
+    if (results[c].state == HIPBLAS_STATUS_SUCCESS && results[c].workspaceSize == 0) {
+      p.algoNoWs = results[c].algo;
+      p.hasNoWs = true;
+    }
+
+  // The kernel: the table, else the rule; a measurement only when asked for.
+  const bool mfmaShape = (dt == DType::F16 || dt == DType::BF16) && M > 0 && M % 128 == 0 && (N % 128 == 0 || N % 96 == 0) && K % 32 == 0;
+  p.handWritten = mfmaShape && ruleSaysHandWritten(M, N, K, act);
+  for (const TableEntry &e : kTable)
+    if (e.dt == (int)dt && e.M == M && e.N == N && e.K == K && e.hasBias == (int)hasBias && e.act == act &&
+        e.hasResidual == (int)hasResidual)
+      p.handWritten = mfmaShape && e.handWritten != 0;
+  if (tune) {
+    const int best = fastestCandidate(p, results, returned, dt, M, N, K, hasBias, act, hasResidual, &p.handWritten);
+    p.algo = results[best].algo;
+    p.algoWorkspace = results[best].workspaceSize;
+  }
   if (forcedKernel()) p.handWritten = forcedKernel() == 2;
   return plans.emplace(key, p).first->second;
 }
@@ -265,15 +326,15 @@ const Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int
 void gemmInit() {
   if (ltHandle) return;
   MGPU_CHECK_BLAS(hipblasLtCreate(&ltHandle));
-  MGPU_CHECK_HIP(hipMalloc(&workspace, workspaceSize));
 }
 
 void gemmDeinit() {
   std::lock_guard<std::mutex> lock(planMutex);
   for (auto &kv : plans) destroyPlan(kv.second);
   plans.clear();
-  if (workspace) (void)hipFree(workspace);
-  workspace = nullptr;
+  for (auto &kv : workspaceOf)
+    if (kv.second) (void)hipFree(kv.second);
+  workspaceOf.clear();
   if (ltHandle) hipblasLtDestroy(ltHandle);
   ltHandle = nullptr;
 }
@@ -293,7 +354,7 @@ void matmulEx(DType dt, const void *input, const void *weight, const void *bias,
     fail("matmul: an activation cannot be combined with a residual");
 
   std::lock_guard<std::mutex> lock(planMutex);
-  const Plan &p = getPlan(dt, M, N, K, hasBias, act, hasResidual, stream);
+  const Plan &p = getPlan(dt, M, N, K, hasBias, act, hasResidual, false);
   if (p.handWritten && gemmMfmaSupports(dt, input, weight, hasBias ? bias : nullptr,
                                         hasResidual ? residual : nullptr, output, M, N, K)) {
     gemmMfma(dt, input, weight, hasBias ? bias : nullptr, hasResidual ? residual : nullptr, output, M, N, K, act,
@@ -304,9 +365,17 @@ void matmulEx(DType dt, const void *input, const void *weight, const void *bias,
     MGPU_CHECK_BLAS(hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias,
                                                     sizeof(bias)));
   const float alpha = 1.0f, beta = hasResidual ? 1.0f : 0.0f;
+  // The stream's own workspace; a stream first met under capture has none and runs the
+  // first algorithm that does without.
+  void *workspace = p.algoWorkspace ? workspaceFor(stream) : nullptr;
+  const hipblasLtMatmulAlgo_t *algo = &p.algo;
+  if (p.algoWorkspace && !workspace) {
+    if (!p.hasNoWs) fail("matmul: the library needs a workspace for this shape; run it once on this stream before capturing");
+    algo = &p.algoNoWs;
+  }
   MGPU_CHECK_BLAS(hipblasLtMatmul(ltHandle, p.op, &alpha, weight, p.a, input, p.b, &beta,
-                                  hasResidual ? residual : output, p.d, output, p.d, &p.algo,
-                                  workspace, workspaceSize, stream));
+                                  hasResidual ? residual : output, p.d, output, p.d, algo,
+                                  workspace, workspace ? workspaceSize : 0, stream));
   if (act == ACT_GELU) {
     if (dt == DType::F16)
       geluInPlaceF16(output, (size_t)M * N, stream);
@@ -315,6 +384,19 @@ void matmulEx(DType dt, const void *input, const void *weight, const void *bias,
     else
       geluInPlaceF32(static_cast<float *>(output), (size_t)M * N, stream);
   }
+}
+
+// Measures, on this device and on scratch operands of the shape, the library's top
+// candidates and the hand-written kernel, and keeps the faster path for the rest of the
+// process.  Synchronous, allocates and frees device memory: never call it under stream
+// capture or from a path that must only enqueue.  Returns true when the hand-written
+// kernel was kept.
+bool tuneMatmulEx(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual) {
+  if (M <= 0 || N <= 0 || K <= 0) fail("tuneMatmulEx: bad shape");
+  if (!ltHandle) fail("tuneMatmulEx: gpuOpsInit() has not been called");
+  if (act < ACT_NONE || act > ACT_GELU || (act != ACT_NONE && hasResidual)) fail("tuneMatmulEx: bad epilogue");
+  std::lock_guard<std::mutex> lock(planMutex);
+  return getPlan(dt, M, N, K, hasBias, act, hasResidual, true).handWritten;
 }
 
 } // namespace mgpu

@@ -30,7 +30,7 @@ namespace mgpu {
 
 namespace {
 
-constexpr size_t kNoAllocScratchBytes = size_t(48) << 20; // 48 MiB: (32,128,768) with ffn 3072 needs 42 MiB
+constexpr size_t kNoAllocScratchBytes = size_t(48) << 20; // 48 MiB: (32,128,768) with ffn 3072 needs 36 MiB
 
 static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
 
@@ -81,19 +81,19 @@ void bertEncoderLayerF16NoAlloc(const void *x, const void *wqkv, const void *bqk
 
   // Layout: [ qkv (3d) | ctx (d) ] shares its bytes with the FFN activation
   // (ffn wide), which is written only after both are dead; then the
-  // projection (reused for the FFN2 output), the residual sum and the first
-  // LayerNorm output.
+  // projection (reused for the FFN2 output) and the first LayerNorm output.
+  // (The rounded residual sums have no reader and are not written.)
   const size_t qkvBytes = roundUp256((size_t)M * 3 * d * h), rowBytes = roundUp256((size_t)M * d * h);
   const size_t ffnBytes = roundUp256((size_t)M * ffn * h);
   const size_t headBytes = qkvBytes + rowBytes > ffnBytes ? qkvBytes + rowBytes : ffnBytes;
-  const size_t need = headBytes + 3 * rowBytes;
+  const size_t need = headBytes + 2 * rowBytes;
   if (need > kNoAllocScratchBytes)
     fail(std::string(name) + ": the layer needs " + std::to_string(need) + " bytes of temporaries, the fixed scratch holds " +
-         std::to_string(kNoAllocScratchBytes) + " (batch * seq_len * (max(4 * d_model, feed_forward_dim) + 3 * d_model) * 2)");
+         std::to_string(kNoAllocScratchBytes) + " (batch * seq_len * (max(4 * d_model, feed_forward_dim) + 2 * d_model) * 2)");
 
   unsigned char *base = scratchOnCurrentDevice();
   void *qkv = base, *ctx = base + qkvBytes, *f = base;
-  void *proj = base + headBytes, *sum = base + headBytes + rowBytes, *h1 = base + headBytes + 2 * rowBytes;
+  void *proj = base + headBytes, *h1 = base + headBytes + rowBytes;
 
   auto gemm = [&](const void *in, const void *w, const void *bias, void *o, int64_t N, int64_t K, int act) {
     if (!gemmMfmaSupports(DType::F16, in, w, bias, nullptr, o, M, N, K))
@@ -106,10 +106,10 @@ void bertEncoderLayerF16NoAlloc(const void *x, const void *wqkv, const void *bqk
   fusedMHA(DType::F16, qkv, seqlens, ctx, (int)B, (int)S, (int)H, (int)(d / H), 1.0f / sqrtf((float)(d / H)), false,
            stream);
   gemm(ctx, wo, bo, proj, d, d, ACT_NONE);
-  layerNorm(DType::F16, proj, x, gamma1, beta1, sum, h1, eps, (int)M, (int)d, stream);
+  layerNorm(DType::F16, proj, x, gamma1, beta1, nullptr, h1, eps, (int)M, (int)d, stream);
   gemm(h1, w1, b1, f, ffn, d, ACT_GELU);
   gemm(f, w2, b2, proj, d, ffn, ACT_NONE);
-  layerNorm(DType::F16, proj, h1, gamma2, beta2, sum, out, eps, (int)M, (int)d, stream);
+  layerNorm(DType::F16, proj, h1, gamma2, beta2, nullptr, out, eps, (int)M, (int)d, stream);
 }
 
 } // namespace mgpu

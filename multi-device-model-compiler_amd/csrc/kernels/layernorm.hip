@@ -107,7 +107,7 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
     const float rstd = 1.0f / sqrtf(var + eps);
 
     u32x4 *yv = reinterpret_cast<u32x4 *>(normed + (size_t)row * n);
-    u32x4 *sv = RESIDUAL ? reinterpret_cast<u32x4 *>(sumOut + (size_t)row * n) : nullptr;
+    u32x4 *sv = (RESIDUAL && sumOut) ? reinterpret_cast<u32x4 *>(sumOut + (size_t)row * n) : nullptr;
 #pragma unroll
     for (int k = 0; k < VPL; k++) {
       const int v = lane + k * LANES;
@@ -119,8 +119,9 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
           // The sum is stored rounded to T and the normalised value is taken
           // from that rounded sum, while mean and variance came from the
           // un-rounded fp32 sums (reference dataflow, LayerNorm.cu:203-233).
+          // (a caller that has no use for the sum passes no buffer for it)
           const u32x4 packed = Tr::pack(x[k]);
-          __builtin_nontemporal_store(packed, sv + v);
+          if (sv) __builtin_nontemporal_store(packed, sv + v);
           Tr::unpack(packed, x[k]);
         }
 #pragma unroll
@@ -343,9 +344,8 @@ __global__ __launch_bounds__(256) void layernorm_block_kernel(
           u32x4 *yv = reinterpret_cast<u32x4 *>(normed + (size_t)(row0 + r) * n);
           float y[VEC];
           if (RESIDUAL) { // rounded sum out, normalised value from the rounded sum (see above)
-            u32x4 *sv = reinterpret_cast<u32x4 *>(sumOut + (size_t)(row0 + r) * n);
             const u32x4 packed = Tr::pack(x[r][k]);
-            __builtin_nontemporal_store(packed, sv + v);
+            if (sumOut) __builtin_nontemporal_store(packed, reinterpret_cast<u32x4 *>(sumOut + (size_t)(row0 + r) * n) + v);
             Tr::unpack(packed, x[r][k]);
           }
 #pragma unroll
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(256) void layernorm_general_kernel(
       float v = value(i);
       if (RESIDUAL) {
         const T rounded = Tr::fromFloat(v);
-        sumOut[(size_t)row * n + i] = rounded;
+        if (sumOut) sumOut[(size_t)row * n + i] = rounded;
         v = Tr::toFloat(rounded);
       }
       normed[(size_t)row * n + i] =
@@ -525,8 +525,7 @@ void layerNorm(DType dt, const void *input, const void *residual, const void *ga
   if (m < 0 || n < 0) fail("layerNorm: negative shape");
   if (m == 0 || n == 0) return;
   if (!input || !gamma || !beta || !normed) fail("layerNorm: null pointer");
-  if ((residual == nullptr) != (sumOut == nullptr))
-    fail("layerNorm: residual and sum output must be given together");
+  if (sumOut && !residual) fail("layerNorm: a sum output needs a residual");
   switch (dt) {
   case DType::F32:
     layerNormDispatch<float>(input, residual, gamma, beta, sumOut, normed, eps, m, n, stream);

@@ -290,7 +290,7 @@ void bertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, cons
 
   Arena arena;
   const size_t oQkv = arena.reserve(M * 3 * d * h), oCtx = arena.reserve(M * d * h);
-  const size_t oProj = arena.reserve(M * d * h), oSum = arena.reserve(M * d * h);
+  const size_t oProj = arena.reserve(M * d * h);
   const size_t oH1 = arena.reserve(M * d * h), oF = arena.reserve(M * ffn * h);
   arena.allocate(stream);
 
@@ -300,13 +300,14 @@ void bertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, cons
            1.0f / sqrtf((float)(d / H)), false, stream);
   matmulEx(DType::F16, arena.at(oCtx), wo, bo, arena.at(oProj), nullptr, M, d, d, true, ACT_NONE,
            false, stream);
-  layerNorm(DType::F16, arena.at(oProj), x, gamma1, beta1, arena.at(oSum), arena.at(oH1), eps,
+  // (nobody reads the rounded sums of this layer: they are not written)
+  layerNorm(DType::F16, arena.at(oProj), x, gamma1, beta1, nullptr, arena.at(oH1), eps,
             (int)M, (int)d, stream);
   matmulEx(DType::F16, arena.at(oH1), w1, b1, arena.at(oF), nullptr, M, ffn, d, true, ACT_GELU,
            false, stream);
   matmulEx(DType::F16, arena.at(oF), w2, b2, arena.at(oProj), nullptr, M, d, ffn, true, ACT_NONE,
            false, stream);
-  layerNorm(DType::F16, arena.at(oProj), arena.at(oH1), gamma2, beta2, arena.at(oSum), out, eps,
+  layerNorm(DType::F16, arena.at(oProj), arena.at(oH1), gamma2, beta2, nullptr, out, eps,
             (int)M, (int)d, stream);
   arena.release(stream);
 }

@@ -14,7 +14,7 @@ enum class DType { F32 = 0, F16 = 1, BF16 = 2 };
 
 void addF32(const float *a, const float *b, float *c, int64_t n, hipStream_t stream);
 
-// residual / sumOut may be null (plain LayerNorm).
+// residual may be null (plain LayerNorm); sumOut may be null (the rounded sum is then not written).
 void layerNorm(DType dt, const void *input, const void *residual, const void *gamma,
                const void *beta, void *sumOut, void *normed, float eps, int m, int n,
                hipStream_t stream);
@@ -59,6 +59,11 @@ void gemmDeinit();
 void matmulEx(DType dt, const void *input, const void *weight, const void *bias, void *output,
               const void *residual, int64_t M, int64_t N, int64_t K, bool hasBias, int act,
               bool hasResidual, hipStream_t stream);
+
+// Explicit, synchronous measurement of a shape (library candidates against the
+// hand-written kernel); the result replaces the table's / the rule's choice for
+// the rest of the process.  Not for capture or enqueue-only paths.
+bool tuneMatmulEx(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual);
 
 // Hand-written MFMA GEMM (gemm_mfma.hip): fp16 / bf16, M a multiple of 128, N of
 // 128 or 96, K of 32, 16-byte aligned operands; bias and residual may be null.

@@ -6,7 +6,13 @@
 //   * the same copy at the grid and byte count of the headline LayerNorm
 //     configuration: the cost of launching, filling and draining 1024 blocks;
 //   * a loop of register-fed v_mfma_f32_32x32x16_f16 on four independent
-//     accumulators, with the shader clock read inside the kernel.
+//     accumulators, with the shader clock read inside the kernel;
+//   * the instruction mix of one 64-key tile of the attention kernel at head_dim
+//     64 (16 MFMAs; per score one fma, one exp2, one add, half a convert; 8
+//     ds_read_b128 and 16 ds_read_b64_tr_b16 whose results nobody waits for),
+//     once finely interleaved and once in the kernel's phases (scores, softmax,
+//     P.V), with no barrier, no tile loads and no wait on LDS data: what a SIMD
+//     can issue for that mix, in shader clocks per tile.
 // Measurement plumbing only: nothing here is part of the kernel library.
 #include <hip/hip_runtime.h>
 
@@ -49,6 +55,75 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float *__restrict__ sin
     stamps[2 * blockIdx.x] = t1 - t0;
     stamps[2 * blockIdx.x + 1] = w1 - w0;
   }
+}
+
+// MODE 0: MFMAs spread evenly through the softmax instructions; 1: eight MFMAs, the
+// softmax, eight MFMAs, each phase fed by the one before (the product kernel's order).
+template <int MODE> __global__ __launch_bounds__(256) void probe_fmha_mix_kernel(float *__restrict__ sink,
+                                                                                 uint64_t *__restrict__ stamps, int tiles) {
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[16384];
+  for (int i = threadIdx.x; i < 4096; i += 256) reinterpret_cast<uint32_t *>(smem)[i] = i;
+  __syncthreads();
+  const uint32_t lbase =
+      (uint32_t)(uintptr_t)((__attribute__((address_space(3))) unsigned char *)smem) + (threadIdx.x % 64) * 16;
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  float a[8];
+  for (int i = 0; i < 8; i++) a[i] = 0.5f + 0.001f * (float)(threadIdx.x + i);
+  f16x8 ma, mb;
+  for (int i = 0; i < 8; i++) {
+    ma[i] = (_Float16)0.01f;
+    mb[i] = (_Float16)0.02f;
+  }
+  f32x16 c0 = {}, c1 = {};
+  u32x4 ra = {0, 0, 0, 0};
+  u32x2 rb = {0, 0};
+  auto softmax8 = [&](int r) { // the softmax instructions of 8 scores
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      asm volatile("v_fma_f32 %0, %0, %0, %0\n v_exp_f32 %0, %0\n v_add_f32 %1, %1, %0" : "+v"(a[i]), "+v"(a[(i + 1) & 7]));
+      if (i & 1) asm volatile("v_cvt_pk_f16_f32 %0, %0, %1" : "+v"(a[i]) : "v"(a[i - 1]));
+      if (MODE == 0) {
+        if (i == 0 || i == 4) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(ra) : "v"(lbase), "i"(r * 2048 + i * 128));
+        if (i & 1) {
+          asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(rb) : "v"(lbase), "i"(r * 2048 + i * 64));
+          if (i & 2) c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma, mb, c0, 0, 0, 0);
+          else c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma, mb, c1, 0, 0, 0);
+        }
+      }
+    }
+  };
+  const uint64_t t0 = clock64();
+  for (int t = 0; t < tiles; t++) {
+    if (MODE == 1) {
+#pragma unroll
+      for (int r = 0; r < 8; r++) {
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(ra) : "v"(lbase), "i"(r * 1024));
+        if (r & 1) c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma, mb, c0, 0, 0, 0);
+        else c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma, mb, c1, 0, 0, 0);
+      }
+      a[0] += c0[0]; // the softmax starts from the scores
+      a[1] += c1[0];
+    }
+#pragma unroll
+    for (int r = 0; r < 4; r++) softmax8(r);
+    if (MODE == 1) {
+      ma[0] = (_Float16)a[0]; // P.V starts from the softmax
+#pragma unroll
+      for (int r = 0; r < 8; r++) {
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(rb) : "v"(lbase), "i"(r * 1024));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(rb) : "v"(lbase), "i"(r * 1024 + 512));
+        if (r & 1) c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma, mb, c0, 0, 0, 0);
+        else c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma, mb, c1, 0, 0, 0);
+      }
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)");
+  const uint64_t t1 = clock64();
+  float s = (float)(ra[0] + rb[0]);
+  for (int i = 0; i < 8; i++) s += a[i];
+  for (int i = 0; i < 16; i++) s += c0[i] + c1[i];
+  if (s == 12345.678f) sink[0] = s;
+  if (threadIdx.x == 0) stamps[blockIdx.x] = t1 - t0;
 }
 
 template <typename F> float timed(F &&launch, int steps, int warmup, hipStream_t stream) {
@@ -100,6 +175,26 @@ float mgpuProbeMfma(void *sink, void *stamps, int blocks, int iters, uint64_t *s
   *shaderClocks = host[0];
   *constClocks = host[1];
   return ms;
+}
+
+// Mean shader clocks per tile and wavefront of the attention instruction mix (mode 0 interleaved,
+// 1 in phases) with `blocks` blocks of four wavefronts; stamps must hold `blocks` uint64.  < 0 on failure.
+double mgpuProbeFmhaMix(void *sink, void *stamps, int blocks, int tiles, int mode, void *stream) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  for (int rep = 0; rep < 2; rep++) {
+    if (mode == 0) probe_fmha_mix_kernel<0><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<float *>(sink), static_cast<uint64_t *>(stamps), tiles);
+    else probe_fmha_mix_kernel<1><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<float *>(sink), static_cast<uint64_t *>(stamps), tiles);
+  }
+  if (hipStreamSynchronize(s) != hipSuccess || hipGetLastError() != hipSuccess) return -1.0;
+  uint64_t *host = new uint64_t[blocks];
+  double mean = -1.0;
+  if (hipMemcpy(host, stamps, sizeof(uint64_t) * blocks, hipMemcpyDeviceToHost) == hipSuccess) {
+    double total = 0.0;
+    for (int i = 0; i < blocks; i++) total += (double)host[i];
+    mean = total / blocks / tiles;
+  }
+  delete[] host;
+  return mean;
 }
 
 // Rate of the constant clock behind wall_clock64(), in kHz (0 if the runtime does not say).
