@@ -25,19 +25,29 @@ import sys
 
 COPY_BYTES = 64 << 20
 
+# (the profiler prints some names demangled and some not: both spellings are matched)
+def fmha(d, causal):
+    c = "true" if causal else "false"
+    return rf"fmha_fwd_kernel(<_Float16, ?{d}, ?\d+, ?{c}|IDF16_Li{d}ELi\d+ELb{int(causal)}E)"
+
+
+# the plain LayerNorm (template argument RESIDUAL = false), not the add-residual form the layers launch
+LN_F32 = r"layernorm_rows_kernel(<float, ?\d+, ?\d+, ?false|IfLi\d+ELi\d+ELb0E)"
+LN_F16 = r"layernorm_rows_kernel(<_Float16, ?\d+, ?\d+, ?false|IDF16_Li\d+ELi\d+ELb0E)"
+
 # bench entry -> (regex on the kernel name, grid size in threads or None for any, algorithmic bytes)
 ENTRIES = {
-    "layernorm_f32": (r"layernorm_rows_kernel<float", 4096 * 64, 25_171_968),
-    "layernorm_f16": (r"layernorm_rows_kernel<_Float16", 4096 * 32, 12_585_984),
+    "layernorm_f32": (LN_F32, 4096 * 64, 25_171_968),
+    "layernorm_f16": (LN_F16, 4096 * 32, 12_585_984),
     "add_f32": (r"add_f32_vec4_kernel", 1200 * 256, 14_745_600),
-    "layernorm_f32_large": (r"layernorm_rows_kernel<float", 262144 * 64, 1_610_618_880),
+    "layernorm_f32_large": (LN_F32, 262144 * 64, 1_610_618_880),
     "add_f32_large": (r"add_f32_vec4_kernel", (1 << 28) // 4, 3_221_225_472),
-    "fmha_b32_s128": (r"fmha_fwd_kernel<_Float16, ?64, ?\d+, ?false>", 32 * 12 * 1 * 256, 25_165_824),
-    "fmha_b8_s512_masked": (r"fmha_fwd_kernel<_Float16, ?64, ?\d+, ?false>", 8 * 16 * 4 * 256, 33_554_464),
-    "fmha_b32_s512": (r"fmha_fwd_kernel<_Float16, ?64, ?\d+, ?false>", 32 * 12 * 4 * 256, 100_663_296),
-    "fmha_b32_s512_causal": (r"fmha_fwd_kernel<_Float16, ?64, ?\d+, ?true>", None, 100_663_296),
-    "fmha_d128_b32_s512": (r"fmha_fwd_kernel<_Float16, ?128, ?\d+, ?false>", 32 * 8 * 4 * 256, 134_217_728),
-    "fmha_d128_b4_s2048": (r"fmha_fwd_kernel<_Float16, ?128, ?\d+, ?false>", 4 * 32 * 16 * 256, 268_435_456),
+    "fmha_b32_s128": (fmha(64, False), 32 * 12 * 1 * 256, 25_165_824),
+    "fmha_b8_s512_masked": (fmha(64, False), 8 * 16 * 4 * 256, 33_554_464),
+    "fmha_b32_s512": (fmha(64, False), 32 * 12 * 4 * 256, 100_663_296),
+    "fmha_b32_s512_causal": (fmha(64, True), None, 100_663_296),
+    "fmha_d128_b32_s512": (fmha(128, False), 32 * 8 * 4 * 256, 134_217_728),
+    "fmha_d128_b4_s2048": (fmha(128, False), 4 * 32 * 16 * 256, 268_435_456),
 }
 COPY_KERNEL = r"copyBuffer"
 
