@@ -40,8 +40,11 @@ extern "C" {
 typedef void *mgpuStream_t; /* hipStream_t */
 
 /* ---- library lifetime (Ops.h:15-18; Ops.cu:43-55; LLM.cu:14-24) ------- */
-/* C names for gpuOpsInit()/gpuOpsDeinit(): create the hipBLASLt handle and its
- * workspace, the side stream + event the layer entry points use for casts. */
+/* C names for gpuOpsInit()/gpuOpsDeinit(): create the hipBLASLt handle and look
+ * up the fixed scratch array of mgpuBertEncoderLayerF16NoAlloc on the current
+ * device.  Everything that depends on the caller's stream (the library's
+ * workspace, the layers' arena, side stream and events) is created on the first
+ * call that uses that stream and returned by the Deinit call. */
 void mgpuOpsInit(void);
 void mgpuOpsDeinit(void);
 /* Returns the message of the most recent failure on the calling thread, or
