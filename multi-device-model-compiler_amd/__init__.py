@@ -324,8 +324,8 @@ ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
 
 
 def matmul_ex(x, w, bias=None, residual=None, act: int = ACT_NONE, stream=None, kernel: str = "auto"):
-    """kernel "auto": the measured choice between the library and the hand-written
-    MFMA kernel; "mfma": the hand-written kernel itself (fp16 / bf16, M a multiple
+    """kernel "auto": mgpuMatmulEx*, i.e. the library or the hand-written MFMA kernel as
+    the committed table and the fixed rule of the library say; "mfma": the hand-written kernel itself (fp16 / bf16, M a multiple
     of 128, N of 128 or 96, K of 32)."""
     import torch
     M, K = x.shape

@@ -243,3 +243,29 @@ def test_fmha_cu_seqlens_packed_rows(pkg, gpu, oracle, rng, lens, max_s, causal,
         seq = bits[cu[b]:cu[b + 1]][None]  # [1, n, 3, H, D]
         ref = oracle.fmha(seq.view(np.float16) if dtype == "f16" else seq, None, causal=causal, bf16=dtype == "bf16")[0]
         assert excess(got[cu[b]:cu[b + 1]], ref, tol) <= 1.0, (b, n)
+
+
+def test_fmha_profile_entry_point_matches_the_product_kernel(pkg, gpu):
+    """mgpuFusedMHAF16Profile is the head_dim-64 kernel with clock stamps: the same
+    output bits as mgpuFusedMHAF16, one record of ten counters per block, stamps in order."""
+    import torch
+    B, S, H, D = 2, 320, 3, 64
+    g = torch.Generator(device=gpu).manual_seed(11)
+    qkv = torch.randn((B, S, 3, H, D), device=gpu, generator=g).half()
+    want = pkg.fused_mha(qkv)
+    out = torch.zeros_like(want)
+    blocks = B * H * ((S + 127) // 128)
+    stamps = torch.zeros(blocks * 10, dtype=torch.int64, device=gpu)
+    lib = pkg.ops()
+    got = lib.mgpuFusedMHAF16Profile(qkv.data_ptr(), out.data_ptr(), B, S, H, D ** -0.5, stamps.data_ptr(),
+                                     torch.cuda.current_stream().cuda_stream)
+    assert lib.mgpuOpsTakeLastError() is None
+    assert got == blocks
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    t = stamps.cpu().numpy().reshape(blocks, 10)
+    entry, first, loop_end, stored, wall0, wall1 = (t[:, i] for i in range(6))
+    assert np.all(entry < first) and np.all(first < loop_end) and np.all(loop_end < stored)
+    assert np.all(wall1 > wall0)
+    phases = t[:, 6:10].sum(axis=1)             # wait + scores + softmax + P.V of all tiles of the block
+    assert np.all(phases > 0) and np.all(phases <= stored - entry)

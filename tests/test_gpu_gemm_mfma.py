@@ -170,3 +170,60 @@ def test_gemm_mfma_refuses_a_misaligned_bias(pkg, gpu):
     b = torch.zeros((130,), dtype=torch.float16, device=gpu)[1:129]   # 2 bytes off the 8-byte grid
     with pytest.raises(pkg.MgpuError):
         pkg.matmul_ex(x, w, bias=b, kernel="mfma")
+
+
+def test_explicit_tuning_keeps_the_results(pkg, gpu, oracle, rng):
+    """mgpuMatmulExTune measures one shape on request (never inside a compute call) and
+    returns which kernel it kept; the GEMM of that shape stays within one fp16 spacing
+    of the oracle whichever it was, and an unusable request reports -1."""
+    M, K, N = 256, 160, 384
+    lib = pkg.ops()
+    kept = lib.mgpuMatmulExTune(1, M, N, K, 1, 0, 1)
+    assert lib.mgpuOpsTakeLastError() is None
+    assert kept in (0, 1)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    b = rng.standard_normal(N).astype(np.float16)
+    r = rng.standard_normal((M, N)).astype(np.float16)
+    got = pkg.matmul_ex(*[to_dev(t, gpu) for t in (x, w, b, r)]).cpu().numpy().astype(np.float32)
+    ref = oracle.gemm(x, w, bias=b, residual=r)
+    assert np.all(np.abs(got - ref) <= spacing_tol(ref, 10, 1e-3))
+    assert lib.mgpuMatmulExTune(7, M, N, K, 1, 0, 1) == -1      # no such element type
+    assert lib.mgpuOpsTakeLastError() is not None
+
+
+def test_library_gemm_captured_on_a_stream_that_has_no_workspace(pkg, gpu, oracle, rng):
+    """The library's workspace belongs to a caller stream and is allocated on that
+    stream's first GEMM outside a capture.  A GEMM captured on a stream that never ran
+    one must not allocate: it takes an algorithm that needs no workspace, and every
+    replay gives the eager result's matrix (fp32: always the library's kernel)."""
+    import torch
+    M, K, N = 96, 200, 72
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    tx, tw, tb = [to_dev(t, gpu) for t in (x, w, b)]
+    out = torch.zeros((M, N), device=gpu)
+    lib = pkg.ops()
+    st = torch.cuda.Stream()                    # fresh: no workspace behind it
+
+    def call():
+        lib.mgpuMatmulExF32(tx.data_ptr(), tw.data_ptr(), tb.data_ptr(), out.data_ptr(), None, M, N, K, 1, 0, 0,
+                            st.cuda_stream)
+        assert lib.mgpuOpsTakeLastError() is None
+
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st):
+        with torch.cuda.graph(graph, stream=st):
+            call()
+    ref = oracle.gemm(x, w, b)
+    for _ in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.abs(out.cpu().numpy() - ref).max() <= 1.2e-5
+    call()                                      # eager, after the capture: may now allocate the workspace
+    st.synchronize()
+    assert np.abs(out.cpu().numpy() - ref).max() <= 1.2e-5
