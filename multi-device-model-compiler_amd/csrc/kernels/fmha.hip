@@ -1,4 +1,5 @@
-// Fused multi-head attention forward for head_dim 64 and 128 on gfx950 MFMA.
+// Fused multi-head attention forward on gfx950 MFMA: tile geometries for head_dim 64 and
+// 128, every other multiple of 8 up to 128 inside the next larger one.
 //
 // Replaces the cubin kernels the reference dispatches through
 // FusedMHARunnerFP16v2 (3rdparty/trt_fused_multihead_attention/
@@ -114,13 +115,20 @@ constexpr float kSumFloor = 0.015625f;
 // exit, and the shader clocks its tiles spent waiting for the tile to land
 // (wait + barrier), in the score MFMAs, in the softmax and in the P.V MFMAs:
 // ten uint64 per block in `stamps`.
-template <typename T, int D, int NQ, bool CAUSAL, bool TRACE = false>
+//
+// PAD: the head dimension in memory, dHead (a multiple of 8 below D), is smaller
+// than the tile geometry D the kernel computes in.  Rows in memory are dHead
+// elements long; a lane whose 16-byte chunk of a K or V row lies beyond dHead
+// fetches chunk 0 of that row instead (in bounds, finite wherever the row is),
+// Q is zero there, so the scores do not see the K filler, and the O^T rows the V
+// filler feeds are never stored.
+template <typename T, int D, int NQ, bool CAUSAL, bool TRACE = false, bool PAD = false>
 __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_kernel(const uint16_t *__restrict__ qkv,
                                                               const int32_t *__restrict__ seqlens,
                                                               const int32_t *__restrict__ cuSeqlens,
                                                               uint16_t *__restrict__ out, int S, int H,
                                                               int nQB, float scale_log2e, int pairItems,
-                                                              uint64_t *__restrict__ stamps) {
+                                                              uint64_t *__restrict__ stamps, int dHead) {
   uint64_t tEntry = 0, wEntry = 0, tFirstTile = 0, tLoopEnd = 0;
   uint64_t cWait = 0, cScores = 0, cSoftmax = 0, cPV = 0, tMark = 0;
   if (TRACE) {
@@ -132,7 +140,9 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   using v4 = typename M::v4;
   using G = Geo<D>;
   constexpr int BM = 128 * NQ;
-  constexpr int kD = D, kBN = G::kBN;
+  constexpr int kBN = G::kBN;
+  const int kD = PAD ? dHead : D;           // elements per head in memory
+  const int validChunks = PAD ? dHead / 8 : G::CPR; // 16-byte chunks of a row that exist
 
   // Ring of kStages stages, each a K tile followed by a V tile; reused as the
   // output staging area at the end.
@@ -207,12 +217,13 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   // 2 KiB of both tiles.  Lane l lands in LDS chunk l % CPR of row l / CPR and
   // fetches global chunk (l % CPR) ^ swizzle(row).
   const int mrow = lane / G::CPR, mchunk = lane % G::CPR;
+  auto srcChunk = [&](int chunk) { return (PAD && chunk >= validChunks) ? 0 : chunk; };
   uint32_t koff[2], voff[2];
 #pragma unroll
   for (int i = 0; i < 2; i++) {
     const int row = G::RPI * (2 * wave + i) + mrow;
-    koff[i] = (uint32_t)row * tokBytes + (uint32_t)((mchunk ^ G::kSwz(row)) * 16);
-    voff[i] = (uint32_t)row * tokBytes + (uint32_t)((mchunk ^ G::vSwz(row)) * 16);
+    koff[i] = (uint32_t)row * tokBytes + (uint32_t)(srcChunk(mchunk ^ G::kSwz(row)) * 16);
+    voff[i] = (uint32_t)row * tokBytes + (uint32_t)(srcChunk(mchunk ^ G::vSwz(row)) * 16);
   }
   // The loads are written as inline assembly so that the compiler's wait-count
   // bookkeeping does not see them: it would otherwise wait for every load in
@@ -249,8 +260,8 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
         int key = kt * kBN + row;
         key = key < rows ? key : rows - 1;
         const uint32_t rowOff = (uint32_t)key * tokBytes;
-        dma16(rowOff + (mchunk ^ G::kSwz(row)) * 16, kbase, kdst + i * 1024);
-        dma16(rowOff + (mchunk ^ G::vSwz(row)) * 16, vbase, vdst + i * 1024);
+        dma16(rowOff + srcChunk(mchunk ^ G::kSwz(row)) * 16, kbase, kdst + i * 1024);
+        dma16(rowOff + srcChunk(mchunk ^ G::vSwz(row)) * 16, vbase, vdst + i * 1024);
       }
     }
   };
@@ -267,8 +278,12 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
     int row = q0 + qi * 32 + l32;
     row = row < rows ? row : rows - 1;
 #pragma unroll
-    for (int c = 0; c < G::DC; c++)
-      qf[qi][c] = *reinterpret_cast<const v8 *>(qbase + (size_t)row * tokBytes + (16 * c + 8 * hl) * 2);
+    for (int c = 0; c < G::DC; c++) {
+      if (!PAD || 2 * c + hl < validChunks)
+        qf[qi][c] = *reinterpret_cast<const v8 *>(qbase + (size_t)row * tokBytes + (16 * c + 8 * hl) * 2);
+      else
+        qf[qi][c] = v8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
   }
 
   // ---- operand addresses inside a stage ---------------------------------------
@@ -486,7 +501,7 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
     const int chunk = it * 64 + lane; // 16-byte chunk index inside the wave's tile
     const int r = chunk / G::CPR, cidx = chunk % G::CPR;
     const int query = q0 + r;
-    if (query < rows) {
+    if (query < rows && (!PAD || cidx < validChunks)) {
       // 8-byte LDS reads: the staging stride is 8-byte but not 16-byte aligned
       const u32x2 lo = *reinterpret_cast<const u32x2 *>(&stage[r * kOS + cidx * 8]);
       const u32x2 hi = *reinterpret_cast<const u32x2 *>(&stage[r * kOS + cidx * 8 + 4]);
@@ -527,9 +542,11 @@ int deviceComputeUnits() {
   return v;
 }
 
-template <typename T, int D, int NQ>
+// dHead: head dimension in memory; D: the tile geometry it runs in (dHead == D, or a
+// smaller multiple of 8 with the PAD instantiation).
+template <typename T, int D, int NQ, bool PAD>
 void launch(const void *qkv, const int32_t *seqlens, const int32_t *cuSeqlens, void *out, int B, int S, int H,
-            float scale, bool causal, hipStream_t stream) {
+            int dHead, float scale, bool causal, hipStream_t stream) {
   constexpr int BM = 128 * NQ;
   const int nQB = (S + BM - 1) / BM;
   // Causal query blocks go in pairs of equal total work when the head dimension
@@ -541,11 +558,24 @@ void launch(const void *qkv, const int32_t *seqlens, const int32_t *cuSeqlens, v
   const float c = scale * 1.44269504088896340736f;
   const auto *in = static_cast<const uint16_t *>(qkv);
   auto *o = static_cast<uint16_t *>(out);
+  const dim3 grid((unsigned)blocks), block(256);
   if (causal)
-    fmha_fwd_kernel<T, D, NQ, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, nullptr);
+    fmha_fwd_kernel<T, D, NQ, true, false, PAD><<<grid, block, 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, nullptr, dHead);
   else
-    fmha_fwd_kernel<T, D, NQ, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, nullptr);
+    fmha_fwd_kernel<T, D, NQ, false, false, PAD><<<grid, block, 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, nullptr, dHead);
   MGPU_CHECK_LAUNCH("fmha_fwd_kernel");
+}
+
+template <typename T>
+void launchForHeadDim(const void *qkv, const int32_t *seqlens, const int32_t *cuSeqlens, void *out, int B, int S, int H,
+                      int dHead, float scale, bool causal, hipStream_t stream) {
+  // One 32-query block per wavefront: 64 queries per wavefront would halve the
+  // LDS operand traffic per flop, but at 224 VGPRs only two wavefronts fit a
+  // SIMD and the kernel measured slower at every shape tried.
+  if (dHead == 64) launch<T, 64, 1, false>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
+  else if (dHead == 128) launch<T, 128, 1, false>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
+  else if (dHead < 64) launch<T, 64, 1, true>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
+  else launch<T, 128, 1, true>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
 }
 
 } // namespace
@@ -554,24 +584,18 @@ namespace {
 void fusedMHAChecked(DType dt, const void *qkv, const int32_t *seqlens, const int32_t *cuSeqlens, void *out, int B,
                      int S, int H, int D, float scale, bool causal, hipStream_t stream) {
   if (B < 0 || S < 0 || H < 0) fail("fusedMHA: negative shape");
-  if (D != 64 && D != 128) fail("fusedMHA: head_dim must be 64 or 128");
+  // 64 and 128 are the tile geometries; the other head sizes of the reference's
+  // dispatcher up to 128 (32, 40, 80; fused_multihead_attention_v2.h:4646-4673) and any
+  // other multiple of 8 run in the next larger geometry with the filler masked out.
+  if (D < 8 || D > 128 || D % 8) fail("fusedMHA: head_dim must be a multiple of 8 between 8 and 128");
   if (B == 0 || S == 0 || H == 0) return;
   if (!qkv || !out) fail("fusedMHA: null pointer");
   if (!aligned16(qkv) || !aligned16(out)) fail("fusedMHA: qkv and out must be 16-byte aligned");
   if (!(scale > 0.0f) || !(scale < INFINITY)) fail("fusedMHA: softmax scale must be positive and finite");
   if ((int64_t)S * 3 * H * D * 2 > 0x7fffffffLL) fail("fusedMHA: one sequence of QKV must stay below 2 GiB");
-  // One 32-query block per wavefront: 64 queries per wavefront would halve the
-  // LDS operand traffic per flop, but at 224 VGPRs only two wavefronts fit a
-  // SIMD and the kernel measured slower at every shape tried.
-  if (dt == DType::F16) {
-    if (D == 64) launch<_Float16, 64, 1>(qkv, seqlens, cuSeqlens, out, B, S, H, scale, causal, stream);
-    else launch<_Float16, 128, 1>(qkv, seqlens, cuSeqlens, out, B, S, H, scale, causal, stream);
-  } else if (dt == DType::BF16) {
-    if (D == 64) launch<bf16_t, 64, 1>(qkv, seqlens, cuSeqlens, out, B, S, H, scale, causal, stream);
-    else launch<bf16_t, 128, 1>(qkv, seqlens, cuSeqlens, out, B, S, H, scale, causal, stream);
-  } else {
-    fail("fusedMHA: element type must be fp16 or bf16");
-  }
+  if (dt == DType::F16) launchForHeadDim<_Float16>(qkv, seqlens, cuSeqlens, out, B, S, H, D, scale, causal, stream);
+  else if (dt == DType::BF16) launchForHeadDim<bf16_t>(qkv, seqlens, cuSeqlens, out, B, S, H, D, scale, causal, stream);
+  else fail("fusedMHA: element type must be fp16 or bf16");
 }
 } // namespace
 
@@ -591,7 +615,7 @@ int64_t fusedMHAProfile(const void *qkv, void *out, int B, int S, int H, float s
   if (blocks > 0x7fffffffLL) fail("fusedMHAProfile: problem too large for one launch");
   fmha_fwd_kernel<_Float16, 64, 1, false, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
       static_cast<const uint16_t *>(qkv), nullptr, nullptr, static_cast<uint16_t *>(out), S, H, nQB,
-      scale * 1.44269504088896340736f, 0, stamps);
+      scale * 1.44269504088896340736f, 0, stamps, 64);
   MGPU_CHECK_LAUNCH("fmha_fwd_kernel (profile)");
   return blocks;
 }

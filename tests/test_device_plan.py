@@ -172,8 +172,8 @@ def test_verifier_messages(tmp_path, body, message):
 
 def test_attention_and_launch_verifiers(tmp_path):
     bad = [
-        ("func @f(%q: 2x16x3x4x32xf16) -> (%o: 2x16x128xf16) {\n  %o = device.fused-mha %q, none : 2x16x128xf16\n  return\n}\n",
-         "head_dim must be 64"),
+        ("func @f(%q: 2x16x3x4x36xf16) -> (%o: 2x16x144xf16) {\n  %o = device.fused-mha %q, none : 2x16x144xf16\n  return\n}\n",
+         "head_dim must be a multiple of 8"),
         ("func @f(%q: 2x16x3x4x64xf32) -> (%o: 2x16x256xf32) {\n  %o = device.fused-mha %q, none : 2x16x256xf32\n  return\n}\n",
          "qkv must be f16 or bf16"),
         ("func @f(%q: 2x16x3x4x64xf16, %l: 3xi32) -> (%o: 2x16x256xf16) {\n  %o = device.fused-mha %q, %l : 2x16x256xf16\n  return\n}\n",

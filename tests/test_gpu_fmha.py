@@ -269,3 +269,43 @@ def test_fmha_profile_entry_point_matches_the_product_kernel(pkg, gpu):
     assert np.all(wall1 > wall0)
     phases = t[:, 6:10].sum(axis=1)             # wait + scores + softmax + P.V of all tiles of the block
     assert np.all(phases > 0) and np.all(phases <= stored - entry)
+
+
+@pytest.mark.parametrize("D,B,S,H,lens,causal,dtype", [
+    (32, 2, 200, 3, None, False, "f16"),       # the reference's kernel list holds 32, 40, 80 next to 64 and 128
+    (40, 2, 257, 2, [257, 90], False, "f16"),
+    (40, 1, 384, 2, None, True, "f16"),         # causal, paired query blocks in the 64-wide geometry
+    (80, 2, 130, 3, [130, 1], False, "f16"),
+    (80, 1, 300, 2, None, True, "bf16"),
+    (96, 2, 96, 2, None, False, "bf16"),
+    (8, 1, 70, 2, None, False, "f16"),          # the smallest head: one 16-byte chunk per row
+    (120, 1, 129, 2, [100], True, "f16"),       # one chunk short of the 128-wide geometry
+])
+def test_fmha_other_head_sizes(pkg, gpu, oracle, rng, D, B, S, H, lens, causal, dtype):
+    """Head sizes between the two tile geometries run inside the next larger one: rows in
+    memory stay D elements long (nothing is padded by the caller), the result is the
+    attention over exactly D dimensions, and no byte outside [B, S, H*D] is written."""
+    import torch
+    qkv = rng.standard_normal((B, S, 3, H, D)).astype(np.float32)
+    tq = torch.from_numpy(qkv).to(gpu).to(torch.float16 if dtype == "f16" else torch.bfloat16)
+    bits = tq.view(torch.int16).cpu().numpy().view(np.uint16)
+    out = torch.full((B * S + 1, H * D), 7.0, dtype=tq.dtype, device=gpu)  # one guard row behind the output
+    tl = to_dev(np.asarray(lens, np.int32), gpu) if lens is not None else None
+    pkg.fused_mha(tq, tl, causal=causal, out=out[:B * S].view(B, S, H * D))
+    got = out.float().cpu().numpy()
+    assert np.all(got[B * S] == 7.0)
+    ref = oracle.fmha(bits.view(np.float16) if dtype == "f16" else bits, lens, causal=causal, bf16=dtype == "bf16")
+    assert excess(got[:B * S].reshape(B, S, H * D), ref, TOL_F16 if dtype == "f16" else TOL_BF16) <= 1.0
+
+
+def test_fmha_other_head_sizes_over_packed_rows(pkg, gpu, oracle, rng):
+    import torch
+    D, H, lens = 40, 2, [70, 0, 200]
+    total = int(np.sum(lens))
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    tq = torch.from_numpy(rng.standard_normal((total, 3, H, D)).astype(np.float32)).to(gpu).half()
+    got = pkg.fused_mha_cu_seqlens(tq, to_dev(cu, gpu), 200).float().cpu().numpy()
+    host = tq.cpu().numpy()
+    for b, n in enumerate(lens):
+        if n:
+            assert excess(got[cu[b]:cu[b + 1]], oracle.fmha(host[cu[b]:cu[b + 1]][None])[0], TOL_F16) <= 1.0, b

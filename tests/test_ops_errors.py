@@ -19,8 +19,8 @@ def take(lib):
 def test_no_error_initially_and_query_clears(lib):
     take(lib)
     assert take(lib) is None
-    lib.mgpuFusedMHAF16(1, None, 1, 1, 1, 1, 32, 0.125, 0, None)
-    assert "head_dim must be 64 or 128" in take(lib)
+    lib.mgpuFusedMHAF16(1, None, 1, 1, 1, 1, 144, 0.125, 0, None)
+    assert "head_dim must be a multiple of 8 between 8 and 128" in take(lib)
     assert take(lib) is None
 
 
@@ -65,7 +65,7 @@ def test_matmul_and_layers_reject_bad_arguments(lib):
     assert "negative" in take(lib)
     lib.mgpuLLMDecodingContextLayer(1, 1, 1, 1, 1, 1, 1, 1, 1, 2, 8, 512, 1024, 8, True, True, True, None)
     assert "gpuOpsInit" in take(lib)
-    lib.mgpuBertEncoderLayerF16(*([1] * 13), None, 1, 2, 8, 768, 3072, 8, 1e-5, None)
-    assert "must be 64" in take(lib)
+    lib.mgpuBertEncoderLayerF16(*([1] * 13), None, 1, 2, 8, 768, 3072, 64, 1e-5, None)
+    assert "multiple of 8 between 8 and 128" in take(lib)
     lib.mgpuAddFusedQKVBiasTransposeF16(16, 16, 16, 16, None, 2, 8, 15, 2, 64, None)
     assert "token_num" in take(lib)
