@@ -97,8 +97,8 @@ void mgpuAddResidualPreLayerNormBF16(const void *input, const void *residual, co
 /* ---- fused multi-head attention -------------------------------------- */
 /* out[b,i,h,:] = sum_j softmax_j(scale * <q[b,i,h,:], k[b,j,h,:]>) v[b,j,h,:]
  * qkv: packed [B, S, 3, H, D]; out: [B, S, H*D]; D is a multiple of 8 between 8
- * and 128 (64 and 128 are the kernel's tile geometries; the other sizes, among
- * them 32, 40 and 80 of the reference's kernel list,
+ * and 256 (64, 128 and 256 are the kernel's tile geometries; the other sizes,
+ * among them 32, 40, 80, 144 and 160 of the reference's kernel list,
  * fused_multihead_attention_v2.h:4646-4673, run inside the next larger one).
  * seqlens: NULL, or B int32 valid key counts (keys j >= seqlens[b] are masked
  * out; all S query rows are produced).  causal != 0 also masks j > i.

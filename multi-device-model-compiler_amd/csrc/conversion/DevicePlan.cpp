@@ -535,7 +535,7 @@ bool verifyOp(const DevicePlan &plan, const DeviceOp &op, std::string &error) {
     const TensorType &q = v.in(0);
     if (q.elem != ElemType::F16 && q.elem != ElemType::BF16) return v.fail("qkv must be f16 or bf16");
     if (q.shape.size() != 5 || q.shape[2] != 3) return v.fail("qkv must be [B, S, 3, H, D]");
-    if (q.shape[4] < 8 || q.shape[4] > 128 || q.shape[4] % 8) return v.fail("head_dim must be a multiple of 8 between 8 and 128");
+    if (q.shape[4] < 8 || q.shape[4] > 256 || q.shape[4] % 8) return v.fail("head_dim must be a multiple of 8 between 8 and 256");
     if (v.present(1)) {
       const TensorType &l = v.in(1);
       if (l.elem != ElemType::I32 || l.shape.size() != 1 || l.shape[0] != q.shape[0]) return v.fail("key lengths must be Bxi32");
@@ -570,7 +570,7 @@ bool verifyOp(const DevicePlan &plan, const DeviceOp &op, std::string &error) {
     auto h = op.attrs.find("head_num");
     if (h == op.attrs.end()) return v.fail("needs head_num");
     const int64_t heads = (int64_t)h->second.number;
-    if (heads <= 0 || d % heads != 0 || d / heads < 8 || d / heads > 128 || (d / heads) % 8) return v.fail("d_model / head_num must be a multiple of 8 between 8 and 128");
+    if (heads <= 0 || d % heads != 0 || d / heads < 8 || d / heads > 256 || (d / heads) % 8) return v.fail("d_model / head_num must be a multiple of 8 between 8 and 256");
     const std::pair<const char *, int64_t> derived[] = {{"batch", x.shape[0]}, {"seq_len", x.shape[1]}, {"d_model", d}, {"feed_forward_dim", ffn}};
     for (const auto &kv : derived) {
       auto a = op.attrs.find(kv.first);
@@ -607,7 +607,7 @@ bool verifyOp(const DevicePlan &plan, const DeviceOp &op, std::string &error) {
     auto h = op.attrs.find("head_num");
     if (h == op.attrs.end()) return v.fail("needs head_num");
     const int64_t heads = (int64_t)h->second.number;
-    if (heads <= 0 || d % heads != 0 || d / heads < 8 || d / heads > 128 || (d / heads) % 8) return v.fail("d_model / head_num must be a multiple of 8 between 8 and 128");
+    if (heads <= 0 || d % heads != 0 || d / heads < 8 || d / heads > 256 || (d / heads) % 8) return v.fail("d_model / head_num must be a multiple of 8 between 8 and 256");
     return true;
   }
   if (n == "gpu.launch_func") {

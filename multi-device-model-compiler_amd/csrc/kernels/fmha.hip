@@ -1,5 +1,5 @@
-// Fused multi-head attention forward on gfx950 MFMA: tile geometries for head_dim 64 and
-// 128, every other multiple of 8 up to 128 inside the next larger one.
+// Fused multi-head attention forward on gfx950 MFMA: tile geometries for head_dim 64,
+// 128 and 256, every other multiple of 8 up to 256 inside the next larger one.
 //
 // Replaces the cubin kernels the reference dispatches through
 // FusedMHARunnerFP16v2 (3rdparty/trt_fused_multihead_attention/
@@ -75,22 +75,32 @@ namespace mgpu {
 
 namespace {
 
-// Geometry per head dimension D (64 or 128).  A K or V tile is always 8 KiB:
-// 64 keys of 128 bytes or 32 keys of 256 bytes, so both share the ring, the
-// movers and the MFMA count per tile (8 for the scores, 8 for P.V); at D = 128
-// a tile carries half as many scores, i.e. half the softmax work per MFMA.
-constexpr int kStages = 3;        // LDS ring depth
-constexpr int kTileBytes = 8192;  // one K or V tile, unpadded rows
+// Geometry per head dimension D (64, 128 or 256).  A K or V tile is 8 KiB at 64 and
+// 128 - 64 keys of 128 bytes or 32 keys of 256 bytes, so both share the movers and
+// the MFMA count per tile (8 for the scores, 8 for P.V); at D = 128 a tile carries
+// half as many scores, i.e. half the softmax work per MFMA.  At D = 256 a tile is
+// 16 KiB (32 keys of 512 bytes, 16 + 16 MFMAs) and the ring has two stages, so that
+// two blocks still share a CU's LDS; their accumulators and Q operands (128 + 64
+// registers) leave room for two wavefronts per SIMD.
 template <int D> struct Geo {
-  static_assert(D == 64 || D == 128, "head dimension 64 or 128");
-  static constexpr int kBN = kTileBytes / (D * 2); // keys per tile: 64 / 32
-  static constexpr int KB = kBN / 32;              // 32-key score blocks per tile: 2 / 1
-  static constexpr int DC = D / 16;                // MFMA k-steps over the head dimension: 4 / 8
-  static constexpr int DB = D / 32;                // 32-row blocks of O^T: 2 / 4
-  static constexpr int rowBytes = D * 2;           // 128 / 256
-  static constexpr int CPR = rowBytes / 16;        // 16-byte chunks per row: 8 / 16
-  static constexpr int RPI = 64 / CPR;             // tile rows one wavefront load instruction fills: 8 / 4
-  static constexpr int OS = D + 4;                 // output staging row stride in elements
+  static_assert(D == 64 || D == 128 || D == 256, "head dimension 64, 128 or 256");
+  static constexpr int kTileBytes = D == 256 ? 16384 : 8192; // one K or V tile, unpadded rows
+  static constexpr int kStages = D == 256 ? 2 : 3;           // LDS ring depth
+  static constexpr int kStageBytes = 2 * kTileBytes;         // a stage: the K tile followed by the V tile
+  static constexpr int LPW = kTileBytes / 4096;     // 1 KiB load instructions per wavefront and tile half: 2 / 2 / 4
+  static constexpr int kBN = kTileBytes / (D * 2);  // keys per tile: 64 / 32 / 32
+  static constexpr int KB = kBN / 32;               // 32-key score blocks per tile: 2 / 1 / 1
+  static constexpr int DC = D / 16;                 // MFMA k-steps over the head dimension: 4 / 8 / 16
+  static constexpr int DB = D / 32;                 // 32-row blocks of O^T: 2 / 4 / 8
+  static constexpr int rowBytes = D * 2;            // 128 / 256 / 512
+  static constexpr int CPR = rowBytes / 16;         // 16-byte chunks per row: 8 / 16 / 32
+  static constexpr int RPI = 64 / CPR;              // tile rows one wavefront load instruction fills: 8 / 4 / 2
+  static constexpr int OS = D + 4;                  // output staging row stride in elements
+  // The swizzles below act on the low four bits of a row's chunk index, so operand
+  // addresses 16 chunks (256 bytes) apart differ by a constant: only KF distinct K
+  // operand addresses and VF distinct V operand addresses are kept in registers.
+  static constexpr int KF = DC < 8 ? DC : 8;
+  static constexpr int VF = DB < 4 ? DB : 4;
   // chunk swizzles (XOR on the 16-byte chunk index of a row) that keep the K
   // operand reads and the transposing V reads free of bank conflicts
   __host__ __device__ static constexpr int kSwz(int row) { return D == 64 ? ((row >> 1) & 7) : (row & 15); }
@@ -141,12 +151,16 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   using G = Geo<D>;
   constexpr int BM = 128 * NQ;
   constexpr int kBN = G::kBN;
+  constexpr int kStages = G::kStages, kTileBytes = G::kTileBytes, kStageBytes = G::kStageBytes, LPW = G::LPW;
   const int kD = PAD ? dHead : D;           // elements per head in memory
   const int validChunks = PAD ? dHead / 8 : G::CPR; // 16-byte chunks of a row that exist
 
   // Ring of kStages stages, each a K tile followed by a V tile; reused as the
-  // output staging area at the end.
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[kStages * 2 * kTileBytes];
+  // output staging area at the end (at D = 256 the staging rows, padded against
+  // bank conflicts, need 1 KiB more than the ring).
+  constexpr int kRingBytes = kStages * kStageBytes;
+  constexpr int kStagingBytes = 4 * NQ * 32 * G::OS * 2;
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[kRingBytes > kStagingBytes ? kRingBytes : kStagingBytes];
 
   // Work-item order: query blocks of one (batch, head) are consecutive, and a
   // contiguous run of work items goes to each of the 8 XCDs (consecutive block
@@ -214,21 +228,21 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
 
   // ---- tile movers: HBM -> LDS, 16 bytes per lane ---------------------------
   // One wavefront instruction fills 1 KiB = RPI tile rows; wavefront w moves
-  // 2 KiB of both tiles.  Lane l lands in LDS chunk l % CPR of row l / CPR and
-  // fetches global chunk (l % CPR) ^ swizzle(row).
+  // a quarter (LPW KiB) of both tiles.  Lane l lands in LDS chunk l % CPR of row
+  // l / CPR and fetches global chunk (l % CPR) ^ swizzle(row).
   const int mrow = lane / G::CPR, mchunk = lane % G::CPR;
   auto srcChunk = [&](int chunk) { return (PAD && chunk >= validChunks) ? 0 : chunk; };
-  uint32_t koff[2], voff[2];
+  uint32_t koff[LPW], voff[LPW];
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
-    const int row = G::RPI * (2 * wave + i) + mrow;
+  for (int i = 0; i < LPW; i++) {
+    const int row = G::RPI * (LPW * wave + i) + mrow;
     koff[i] = (uint32_t)row * tokBytes + (uint32_t)(srcChunk(mchunk ^ G::kSwz(row)) * 16);
     voff[i] = (uint32_t)row * tokBytes + (uint32_t)(srcChunk(mchunk ^ G::vSwz(row)) * 16);
   }
   // The loads are written as inline assembly so that the compiler's wait-count
   // bookkeeping does not see them: it would otherwise wait for every load in
   // flight, prefetches included, before any later LDS read.  Completion is
-  // tracked by hand with s_waitcnt vmcnt(n) below (4 loads per tile and wave).
+  // tracked by hand with s_waitcnt vmcnt(n) below (2 * LPW loads per tile and wave).
   const uint32_t ldsBase = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) unsigned char *)smem);
   // M0 is on the clobber list so that the statement counts as a definition of it
   // (the compiler reserves M0 and notes that such a clobber is not saved and restored:
@@ -243,20 +257,20 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   };
 #pragma clang diagnostic pop
   auto issueTile = [&](int kt) {
-    const uint32_t kdst = ldsBase + (uint32_t)((kt % kStages) * (2 * kTileBytes) + (2 * wave) * 1024);
+    const uint32_t kdst = ldsBase + (uint32_t)((kt % kStages) * kStageBytes + (LPW * wave) * 1024);
     const uint32_t vdst = kdst + kTileBytes;
     if (kt * kBN + kBN <= rows) { // whole tile inside the sequence
       const char *kg = kbase + (size_t)kt * kBN * tokBytes;
       const char *vg = vbase + (size_t)kt * kBN * tokBytes;
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
+      for (int i = 0; i < LPW; i++) {
         dma16(koff[i], kg, kdst + i * 1024);
         dma16(voff[i], vg, vdst + i * 1024);
       }
     } else { // last tile of a ragged sequence: clamp the row, the mask hides it
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
-        const int row = G::RPI * (2 * wave + i) + mrow;
+      for (int i = 0; i < LPW; i++) {
+        const int row = G::RPI * (LPW * wave + i) + mrow;
         int key = kt * kBN + row;
         key = key < rows ? key : rows - 1;
         const uint32_t rowOff = (uint32_t)key * tokBytes;
@@ -288,16 +302,18 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
 
   // ---- operand addresses inside a stage ---------------------------------------
   // K: lane (key l32 [+32kb], d chunk 2c+hl) reads 16 bytes.
-  uint32_t kfrag[G::DC];
+  // (k-steps 8 apart read chunks 16 apart: the swizzle leaves that bit alone)
+  uint32_t kfrag[G::KF];
 #pragma unroll
-  for (int c = 0; c < G::DC; c++) kfrag[c] = (uint32_t)(l32 * G::rowBytes + (((2 * c + hl) ^ G::kSwz(l32)) * 16));
+  for (int c = 0; c < G::KF; c++) kfrag[c] = (uint32_t)(l32 * G::rowBytes + (((2 * c + hl) ^ G::kSwz(l32)) * 16));
   // V: as a source of the transposing read, lane L of a 16-lane group g points
   // at key 4*hl + L/4 (+ 32kb + 16m + 8e), d = 32db + 16*(g%2) + 4*(L%4).
-  uint32_t vfrag[G::DB];
+  // (O^T blocks 4 apart read chunks 16 apart)
+  uint32_t vfrag[G::VF];
   {
     const int g = lane / 16, L = lane % 16, r = L % 4, j = L / 4;
 #pragma unroll
-    for (int db = 0; db < G::DB; db++) {
+    for (int db = 0; db < G::VF; db++) {
       const int chunk = (4 * db + 2 * (g % 2) + r / 2) ^ G::vSwz(4 * hl + j);
       vfrag[db] = (uint32_t)((4 * hl + j) * G::rowBytes + chunk * 16 + 8 * (r % 2));
     }
@@ -320,13 +336,14 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
     // The loads of tile kt (and of nothing later) must have landed; the barrier
     // makes every wavefront's share visible and also says that everybody is
     // done with tile kt-1, whose stage the next load may overwrite.
-    if (kt + 1 < nkt) asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); // vmcnt(4): tile kt+1 may still fly
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");              // vmcnt(0)
+    // (with a ring of three, tile kt + 1 may still fly: its 2 * LPW loads)
+    if (kStages > 2 && kt + 1 < nkt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LPW) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (TRACE && kt == 0) tFirstTile = clock64();
     if (kt + kStages - 1 < nkt) issueTile(kt + kStages - 1);
 
-    const uint32_t stageOff = (uint32_t)((kt % kStages) * (2 * kTileBytes));
+    const uint32_t stageOff = (uint32_t)((kt % kStages) * kStageBytes);
     const int key0 = kt * kBN;
 
     // Rows of masked keys meet p = 0; zero them so that stray NaN/Inf bits in
@@ -334,7 +351,7 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
     if (key0 + kBN > kvlen) {
       unsigned char *vst = smem + stageOff + kTileBytes;
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
+      for (int i = 0; i < kTileBytes / 4096; i++) {
         const int chunk = tid + 256 * i; // 16-byte chunk of the V tile
         if (key0 + chunk / G::CPR >= kvlen)
           *reinterpret_cast<u32x4 *>(vst + chunk * 16) = u32x4{0u, 0u, 0u, 0u};
@@ -347,11 +364,11 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
 
     // Operand pointers in the LDS address space: one add per tile, the rest
     // of every address is an instruction immediate.
-    const lds_u8 *kp[G::DC], *vp[G::DB];
+    const lds_u8 *kp[G::KF], *vp[G::VF];
 #pragma unroll
-    for (int c = 0; c < G::DC; c++) kp[c] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kfrag[c]);
+    for (int c = 0; c < G::KF; c++) kp[c] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kfrag[c]);
 #pragma unroll
-    for (int db = 0; db < G::DB; db++) vp[db] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kTileBytes + vfrag[db]);
+    for (int db = 0; db < G::VF; db++) vp[db] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kTileBytes + vfrag[db]);
 
     if (TRACE) {
       const uint64_t t = clock64();
@@ -365,7 +382,8 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
     for (int kb = 0; kb < G::KB; kb++) {
 #pragma unroll
       for (int c = 0; c < G::DC; c++) {
-        const v8 a = *reinterpret_cast<const v8 __attribute__((address_space(3))) *>(kp[c] + kb * 32 * G::rowBytes);
+        const v8 a = *reinterpret_cast<const v8 __attribute__((address_space(3))) *>(kp[c % G::KF] + (c / G::KF) * 256 +
+                                                                                      kb * 32 * G::rowBytes);
 #pragma unroll
         for (int qi = 0; qi < NQ; qi++) {
           if (c == 0) {
@@ -458,7 +476,7 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
       for (int kb = 0; kb < G::KB; kb++) {
 #pragma unroll
         for (int m = 0; m < 2; m++) {
-          const lds_u8 *p = vp[db] + (32 * kb + 16 * m) * G::rowBytes;
+          const lds_u8 *p = vp[db % G::VF] + (db / G::VF) * 256 + (32 * kb + 16 * m) * G::rowBytes;
           const v4 lo = M::readTr(p);                    // k-slots 0..3: keys +4hl+0..3
           const v4 hi = M::readTr(p + 8 * G::rowBytes);  // k-slots 4..7: keys +8+4hl+0..3
           const v8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -479,7 +497,6 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   __syncthreads(); // every wavefront is done reading the K / V tiles
   constexpr int kOS = G::OS;
   uint16_t *stage = reinterpret_cast<uint16_t *>(smem) + wave * (NQ * 32 * kOS);
-  static_assert(4 * NQ * 32 * kOS * 2 <= kStages * 2 * kTileBytes, "output staging must fit in the ring");
 #pragma unroll
   for (int qi = 0; qi < NQ; qi++) {
     const float l = halves_sum(l_run[qi]);
@@ -574,8 +591,10 @@ void launchForHeadDim(const void *qkv, const int32_t *seqlens, const int32_t *cu
   // SIMD and the kernel measured slower at every shape tried.
   if (dHead == 64) launch<T, 64, 1, false>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
   else if (dHead == 128) launch<T, 128, 1, false>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
+  else if (dHead == 256) launch<T, 256, 1, false>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
   else if (dHead < 64) launch<T, 64, 1, true>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
-  else launch<T, 128, 1, true>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
+  else if (dHead < 128) launch<T, 128, 1, true>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
+  else launch<T, 256, 1, true>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
 }
 
 } // namespace
@@ -584,10 +603,10 @@ namespace {
 void fusedMHAChecked(DType dt, const void *qkv, const int32_t *seqlens, const int32_t *cuSeqlens, void *out, int B,
                      int S, int H, int D, float scale, bool causal, hipStream_t stream) {
   if (B < 0 || S < 0 || H < 0) fail("fusedMHA: negative shape");
-  // 64 and 128 are the tile geometries; the other head sizes of the reference's
-  // dispatcher up to 128 (32, 40, 80; fused_multihead_attention_v2.h:4646-4673) and any
+  // 64, 128 and 256 are the tile geometries; the other head sizes of the reference's
+  // dispatcher (32, 40, 80, 144, 160; fused_multihead_attention_v2.h:4646-4673) and any
   // other multiple of 8 run in the next larger geometry with the filler masked out.
-  if (D < 8 || D > 128 || D % 8) fail("fusedMHA: head_dim must be a multiple of 8 between 8 and 128");
+  if (D < 8 || D > 256 || D % 8) fail("fusedMHA: head_dim must be a multiple of 8 between 8 and 256");
   if (B == 0 || S == 0 || H == 0) return;
   if (!qkv || !out) fail("fusedMHA: null pointer");
   if (!aligned16(qkv) || !aligned16(out)) fail("fusedMHA: qkv and out must be 16-byte aligned");

@@ -71,8 +71,8 @@ void bertEncoderLayerF16NoAlloc(const void *x, const void *wqkv, const void *bqk
                                 hipStream_t stream) {
   const char *name = "mgpuBertEncoderLayerF16NoAlloc";
   if (B < 0 || S < 0 || d <= 0 || ffn <= 0 || H <= 0) fail(std::string(name) + ": bad shape");
-  if (d % H || d / H < 8 || d / H > 128 || (d / H) % 8)
-    fail(std::string(name) + ": d_model / head_num must be a multiple of 8 between 8 and 128");
+  if (d % H || d / H < 8 || d / H > 256 || (d / H) % 8)
+    fail(std::string(name) + ": d_model / head_num must be a multiple of 8 between 8 and 256");
   if (B == 0 || S == 0) return;
   if (!x || !wqkv || !bqkv || !wo || !bo || !gamma1 || !beta1 || !w1 || !b1 || !w2 || !b2 || !gamma2 || !beta2 || !out)
     fail(std::string(name) + ": null pointer");

@@ -174,8 +174,8 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
   if (!initialised) fail("mgpuLLMDecodingContextLayer: gpuOpsInit() has not been called");
   if (batch < 0 || seq_len < 0 || d_model <= 0 || ffn <= 0 || heads <= 0)
     fail("mgpuLLMDecodingContextLayer: bad shape");
-  if (d_model % heads || d_model / heads < 8 || d_model / heads > 128 || (d_model / heads) % 8)
-    fail("mgpuLLMDecodingContextLayer: d_model / head_num must be a multiple of 8 between 8 and 128");
+  if (d_model % heads || d_model / heads < 8 || d_model / heads > 256 || (d_model / heads) % 8)
+    fail("mgpuLLMDecodingContextLayer: d_model / head_num must be a multiple of 8 between 8 and 256");
   if (batch == 0 || seq_len == 0) return;
   if (!input || !qkv || !gemm_weight || !gemm_bias || !ffn1_weight || !ffn1_bias || !ffn2_weight ||
       !ffn2_bias || !output)
@@ -279,8 +279,8 @@ void bertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, cons
                          int64_t S, int64_t d, int64_t ffn, int64_t H, float eps,
                          hipStream_t stream) {
   if (B < 0 || S < 0 || d <= 0 || ffn <= 0 || H <= 0) fail("mgpuBertEncoderLayerF16: bad shape");
-  if (d % H || d / H < 8 || d / H > 128 || (d / H) % 8)
-    fail("mgpuBertEncoderLayerF16: d_model / head_num must be a multiple of 8 between 8 and 128");
+  if (d % H || d / H < 8 || d / H > 256 || (d / H) % 8)
+    fail("mgpuBertEncoderLayerF16: d_model / head_num must be a multiple of 8 between 8 and 256");
   if (B == 0 || S == 0) return;
   if (!x || !wqkv || !bqkv || !wo || !bo || !gamma1 || !beta1 || !w1 || !b1 || !w2 || !b2 ||
       !gamma2 || !beta2 || !out)

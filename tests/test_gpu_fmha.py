@@ -280,9 +280,17 @@ def test_fmha_profile_entry_point_matches_the_product_kernel(pkg, gpu):
     (96, 2, 96, 2, None, False, "bf16"),
     (8, 1, 70, 2, None, False, "f16"),          # the smallest head: one 16-byte chunk per row
     (120, 1, 129, 2, [100], True, "f16"),       # one chunk short of the 128-wide geometry
+    (256, 2, 200, 2, None, False, "f16"),       # the widest head of the reference's kernel list: its own geometry
+    (256, 1, 257, 2, [200], True, "f16"),
+    (256, 2, 96, 3, [96, 33], False, "bf16"),
+    (144, 2, 130, 2, [130, 7], False, "f16"),   # 144 and 160 of the list, inside the 256-wide geometry
+    (160, 1, 300, 3, None, True, "f16"),
+    (160, 2, 64, 2, None, False, "bf16"),
+    (136, 1, 65, 1, None, False, "f16"),        # the first size past the 128-wide geometry
+    (248, 1, 129, 2, [129], True, "f16"),       # one chunk short of the 256-wide geometry
 ])
 def test_fmha_other_head_sizes(pkg, gpu, oracle, rng, D, B, S, H, lens, causal, dtype):
-    """Head sizes between the two tile geometries run inside the next larger one: rows in
+    """Head sizes between the tile geometries (64, 128, 256) run inside the next larger one: rows in
     memory stay D elements long (nothing is padded by the caller), the result is the
     attention over exactly D dimensions, and no byte outside [B, S, H*D] is written."""
     import torch

@@ -19,8 +19,8 @@ def take(lib):
 def test_no_error_initially_and_query_clears(lib):
     take(lib)
     assert take(lib) is None
-    lib.mgpuFusedMHAF16(1, None, 1, 1, 1, 1, 144, 0.125, 0, None)
-    assert "head_dim must be a multiple of 8 between 8 and 128" in take(lib)
+    lib.mgpuFusedMHAF16(1, None, 1, 1, 1, 1, 264, 0.125, 0, None)
+    assert "head_dim must be a multiple of 8 between 8 and 256" in take(lib)
     assert take(lib) is None
 
 
@@ -59,6 +59,13 @@ def test_layernorm_and_add_reject_bad_arguments(lib):
 
 
 def test_matmul_and_layers_reject_bad_arguments(lib):
+    # The calls below hand the library made-up pointers and count on it refusing them before
+    # any launch because gpuOpsInit() has not run.  Ask that with null pointers first: where
+    # another test of this process has initialised the library, the answer is "null pointer"
+    # and the made-up pointers stay out of it.
+    lib.mgpuMatmulExF16(None, None, None, None, None, 4, 4, 4, 0, 0, 0, None)
+    if "gpuOpsInit" not in (take(lib) or ""):
+        pytest.skip("the kernel library is already initialised in this process")
     lib.mgpuMatmulExF16(1, 1, None, 1, None, 4, 4, 4, 0, 0, 0, None)
     assert "gpuOpsInit" in take(lib)  # library not initialised in this process
     lib.mgpuMatmulExF16(1, 1, None, 1, None, -4, 4, 4, 0, 0, 0, None)
@@ -66,6 +73,6 @@ def test_matmul_and_layers_reject_bad_arguments(lib):
     lib.mgpuLLMDecodingContextLayer(1, 1, 1, 1, 1, 1, 1, 1, 1, 2, 8, 512, 1024, 8, True, True, True, None)
     assert "gpuOpsInit" in take(lib)
     lib.mgpuBertEncoderLayerF16(*([1] * 13), None, 1, 2, 8, 768, 3072, 64, 1e-5, None)
-    assert "multiple of 8 between 8 and 128" in take(lib)
+    assert "multiple of 8 between 8 and 256" in take(lib)
     lib.mgpuAddFusedQKVBiasTransposeF16(16, 16, 16, 16, None, 2, 8, 15, 2, 64, None)
     assert "token_num" in take(lib)
