@@ -395,20 +395,45 @@ def measure_ceilings(torch, loops, dev, gen, sp, ptrs, repeats) -> dict:
                                 "what": "v_mfma_f32_32x32x16_f16 on four independent accumulators from registers, "
                                         "4096 x 4 per wavefront, every SIMD of the device; shader clock from clock64() "
                                         "against the constant-rate wall_clock64()"}
-    mix = {}
-    for mode, name in ((0, "interleaved"), (1, "in_phases")):
-        per = {}
-        for waves_per_simd in (1, 2, 3, 4):
-            c = loops.mgpuProbeFmhaMix(ctypes.c_void_p(sink.data_ptr()), ctypes.c_void_p(stamps.data_ptr()),
-                                       256 * waves_per_simd, 400, mode, sp)
-            if c > 0:
-                per[str(waves_per_simd)] = round(c / waves_per_simd, 1)
-        mix[name] = per
-    res["fmha_d64_tile_instruction_mix"] = {
-        "simd_clocks_per_tile_by_wavefronts_per_simd": mix, "mfma_clocks_per_tile": 16 * 32,
-        "what": "the instructions of one 64-key x 32-query tile of the head_dim-64 attention kernel (16 MFMAs, 32 fma / exp2 / "
-                "add, 16 converts, 24 LDS operand reads whose data nobody waits for), no barrier, no tile loads: the clocks a "
-                "SIMD needs per tile for that mix, finely interleaved and in the kernel's three phases"}
+    # the attention tile loop without its bookkeeping (csrc/tools/bench_probes.hip: probe_fmha_loop_kernel)
+    kv = (torch.randn((512, 3, 384, 64), device=dev, generator=None) / 8).half()
+    stamps = torch.zeros(8 * 256 * 3, dtype=torch.int64, device=dev)
+    tiles = 1500
+    model = []
+    names = {0: "three phases per tile", 1: "half-tile pipeline"}
+    for queries, waves_per_simd in ((32, 1), (32, 2), (32, 3), (64, 1), (64, 2)):
+        for pipelined in (0, 1):
+            for loads in (0, 1):
+                variant = pipelined | (2 if queries == 64 else 0) | (4 if loads else 0)
+                blocks = 256 * waves_per_simd
+                best = None
+                for _ in range(2):
+                    sc, cc = ctypes.c_double(0), ctypes.c_double(0)
+                    ms = loops.mgpuProbeFmhaLoop(ctypes.c_void_p(sink.data_ptr()), ctypes.c_void_p(stamps.data_ptr()),
+                                                 ctypes.c_void_p(kv.data_ptr()), blocks, tiles, variant, ctypes.byref(sc),
+                                                 ctypes.byref(cc), sp)
+                    if ms > 0 and (best is None or ms < best[0]):
+                        best = (ms, sc.value, cc.value)
+                if not best:
+                    continue
+                ms, sc, cc = best
+                units = queries // 32                      # 32-query blocks per wavefront
+                flop = blocks * 4.0 * tiles * units * 16 * 32 * 32 * 16 * 2
+                model.append({"queries_per_wavefront": queries, "wavefronts_per_simd": waves_per_simd,
+                              "schedule": names[pipelined], "tile_loads_and_barrier": bool(loads),
+                              "simd_clocks_per_32_query_tile": round(sc / tiles / waves_per_simd / units, 1),
+                              "shader_clock_ghz_in_kernel": round(sc / cc * khz / 1e6, 3) if cc and khz else None,
+                              "TFLOP/s": round(flop / ms / 1e9, 1)})
+    del kv
+    res["fmha_d64_tile_loop_model"] = {
+        "runs": model, "mfma_clocks_per_32_query_tile": 16 * 32,
+        "what": "the tile loop of the head_dim-64 attention kernel without masks, repair path, prologue and epilogue: per "
+                "64-key tile and 32 queries 8 score MFMAs fed by ds_read_b128 of a K tile, the softmax of their results (per "
+                "score one fma, one exp2, one add, half a convert), 8 P.V MFMAs fed by the converted scores and "
+                "ds_read_b64_tr_b16 of a V tile; in the product kernel's three phases or with every MFMA followed by an "
+                "eighth of a half softmax (operand reads three MFMAs ahead); optionally with the product's four "
+                "global_load_lds per wavefront and tile and its block barrier; shader clock from clock64() against "
+                "wall_clock64(), TFLOP/s from the launch's wall time"}
     return res
 
 
@@ -440,7 +465,7 @@ def main():
         for fn in ("mgpuBenchLayerNormF32", "mgpuBenchLayerNormF16", "mgpuBenchAddF32", "mgpuBenchFusedMHAF16",
                    "mgpuBenchBertEncoderLayerF16", "mgpuProbeCopy", "mgpuProbeMfma"):
             getattr(loops, fn).restype = ctypes.c_float
-        loops.mgpuProbeFmhaMix.restype = ctypes.c_double
+        loops.mgpuProbeFmhaLoop.restype = ctypes.c_float
     bench_stream = torch.cuda.Stream()
 
     def ptrs(tensors):

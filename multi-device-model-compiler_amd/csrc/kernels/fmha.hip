@@ -232,12 +232,22 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   // l / CPR and fetches global chunk (l % CPR) ^ swizzle(row).
   const int mrow = lane / G::CPR, mchunk = lane % G::CPR;
   auto srcChunk = [&](int chunk) { return (PAD && chunk >= validChunks) ? 0 : chunk; };
+  // Offsets of this lane's loads inside a tile.  Where registers are short (D = 256)
+  // they are recomputed at every use from the lane's row and chunk - the copy that
+  // goes through the empty asm statement keeps the compiler from hoisting the
+  // arithmetic out of the tile loop and spilling its results instead.
+  constexpr bool kRecomputeOffsets = D == 256;
+  auto tileOffset = [&](int i, bool isV) {
+    int mr = mrow;
+    if (kRecomputeOffsets) asm volatile("" : "+v"(mr));
+    const int row = G::RPI * (LPW * wave + i) + mr;
+    return (uint32_t)row * tokBytes + (uint32_t)(srcChunk(mchunk ^ (isV ? G::vSwz(row) : G::kSwz(row))) * 16);
+  };
   uint32_t koff[LPW], voff[LPW];
 #pragma unroll
   for (int i = 0; i < LPW; i++) {
-    const int row = G::RPI * (LPW * wave + i) + mrow;
-    koff[i] = (uint32_t)row * tokBytes + (uint32_t)(srcChunk(mchunk ^ G::kSwz(row)) * 16);
-    voff[i] = (uint32_t)row * tokBytes + (uint32_t)(srcChunk(mchunk ^ G::vSwz(row)) * 16);
+    koff[i] = kRecomputeOffsets ? 0u : tileOffset(i, false);
+    voff[i] = kRecomputeOffsets ? 0u : tileOffset(i, true);
   }
   // The loads are written as inline assembly so that the compiler's wait-count
   // bookkeeping does not see them: it would otherwise wait for every load in
@@ -264,8 +274,8 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
       const char *vg = vbase + (size_t)kt * kBN * tokBytes;
 #pragma unroll
       for (int i = 0; i < LPW; i++) {
-        dma16(koff[i], kg, kdst + i * 1024);
-        dma16(voff[i], vg, vdst + i * 1024);
+        dma16(kRecomputeOffsets ? tileOffset(i, false) : koff[i], kg, kdst + i * 1024);
+        dma16(kRecomputeOffsets ? tileOffset(i, true) : voff[i], vg, vdst + i * 1024);
       }
     } else { // last tile of a ragged sequence: clamp the row, the mask hides it
 #pragma unroll
@@ -303,21 +313,23 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   // ---- operand addresses inside a stage ---------------------------------------
   // K: lane (key l32 [+32kb], d chunk 2c+hl) reads 16 bytes.
   // (k-steps 8 apart read chunks 16 apart: the swizzle leaves that bit alone)
-  uint32_t kfrag[G::KF];
-#pragma unroll
-  for (int c = 0; c < G::KF; c++) kfrag[c] = (uint32_t)(l32 * G::rowBytes + (((2 * c + hl) ^ G::kSwz(l32)) * 16));
+  auto kfragOf = [&](int c, int row32, int half) {
+    return (uint32_t)(row32 * G::rowBytes + (((2 * c + half) ^ G::kSwz(row32)) * 16));
+  };
   // V: as a source of the transposing read, lane L of a 16-lane group g points
   // at key 4*hl + L/4 (+ 32kb + 16m + 8e), d = 32db + 16*(g%2) + 4*(L%4).
   // (O^T blocks 4 apart read chunks 16 apart)
-  uint32_t vfrag[G::VF];
-  {
-    const int g = lane / 16, L = lane % 16, r = L % 4, j = L / 4;
+  auto vfragOf = [&](int db, int ln) {
+    const int g = ln / 16, L = ln % 16, r = L % 4, j = L / 4, half = ln / 32;
+    const int chunk = (4 * db + 2 * (g % 2) + r / 2) ^ G::vSwz(4 * half + j);
+    return (uint32_t)((4 * half + j) * G::rowBytes + chunk * 16 + 8 * (r % 2));
+  };
+  // (as with the movers' offsets: kept in registers, or recomputed per tile at D = 256)
+  uint32_t kfrag[G::KF], vfrag[G::VF];
 #pragma unroll
-    for (int db = 0; db < G::VF; db++) {
-      const int chunk = (4 * db + 2 * (g % 2) + r / 2) ^ G::vSwz(4 * hl + j);
-      vfrag[db] = (uint32_t)((4 * hl + j) * G::rowBytes + chunk * 16 + 8 * (r % 2));
-    }
-  }
+  for (int c = 0; c < G::KF; c++) kfrag[c] = kRecomputeOffsets ? 0u : kfragOf(c, l32, hl);
+#pragma unroll
+  for (int db = 0; db < G::VF; db++) vfrag[db] = kRecomputeOffsets ? 0u : vfragOf(db, lane);
 
   f32x16 accO[NQ][G::DB];
   float m_run[NQ], l_run[NQ]; // stale reference maximum (raw score units), this lane's share of the running sum
@@ -365,10 +377,14 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
     // Operand pointers in the LDS address space: one add per tile, the rest
     // of every address is an instruction immediate.
     const lds_u8 *kp[G::KF], *vp[G::VF];
+    int ln = lane;
+    if (kRecomputeOffsets) asm volatile("" : "+v"(ln));
 #pragma unroll
-    for (int c = 0; c < G::KF; c++) kp[c] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kfrag[c]);
+    for (int c = 0; c < G::KF; c++)
+      kp[c] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + (kRecomputeOffsets ? kfragOf(c, ln % 32, ln / 32) : kfrag[c]));
 #pragma unroll
-    for (int db = 0; db < G::VF; db++) vp[db] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kTileBytes + vfrag[db]);
+    for (int db = 0; db < G::VF; db++)
+      vp[db] = (const lds_u8 *)(uintptr_t)(ldsBase + stageOff + kTileBytes + (kRecomputeOffsets ? vfragOf(db, ln) : vfrag[db]));
 
     if (TRACE) {
       const uint64_t t = clock64();

@@ -7,12 +7,17 @@
 //     configuration: the cost of launching, filling and draining 1024 blocks;
 //   * a loop of register-fed v_mfma_f32_32x32x16_f16 on four independent
 //     accumulators, with the shader clock read inside the kernel;
-//   * the instruction mix of one 64-key tile of the attention kernel at head_dim
-//     64 (16 MFMAs; per score one fma, one exp2, one add, half a convert; 8
-//     ds_read_b128 and 16 ds_read_b64_tr_b16 whose results nobody waits for),
-//     once finely interleaved and once in the kernel's phases (scores, softmax,
-//     P.V), with no barrier, no tile loads and no wait on LDS data: what a SIMD
-//     can issue for that mix, in shader clocks per tile.
+//   * a model of the attention kernel's tile loop at head_dim 64: the real data
+//     flow of a 64-key tile (eight score MFMAs fed by ds_read_b128 of a K tile,
+//     the softmax of their results - per score one fma, one exp2, one add, half
+//     a convert -, eight P.V MFMAs fed by the converted scores and by
+//     ds_read_b64_tr_b16 of a V tile), in the product kernel's three phases or
+//     as a half-tile software pipeline with every MFMA followed by an eighth of
+//     a half softmax, with 32 or 64 queries per wavefront, with and without the
+//     product's tile loads (global_load_lds into a ring of three) and block
+//     barrier.  No masks, no row-maximum repair, no prologue or epilogue: what
+//     the SIMD, the LDS and the clock governor leave of the matrix rate for this
+//     mix, in shader clocks per tile and in wall-clock TFLOP/s.
 // Measurement plumbing only: nothing here is part of the kernel library.
 #include <hip/hip_runtime.h>
 
@@ -57,73 +62,217 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float *__restrict__ sin
   }
 }
 
-// MODE 0: MFMAs spread evenly through the softmax instructions; 1: eight MFMAs, the
-// softmax, eight MFMAs, each phase fed by the one before (the product kernel's order).
-template <int MODE> __global__ __launch_bounds__(256) void probe_fmha_mix_kernel(float *__restrict__ sink,
-                                                                                 uint64_t *__restrict__ stamps, int tiles) {
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[16384];
-  for (int i = threadIdx.x; i < 4096; i += 256) reinterpret_cast<uint32_t *>(smem)[i] = i;
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned char __attribute__((address_space(3))) lds_u8;
+
+__device__ __forceinline__ f16x4 probeReadTr(const lds_u8 *p) {
+  return __builtin_bit_cast(f16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 __attribute__((address_space(3))) *)p));
+}
+__device__ __forceinline__ f32x16 probeMfma(f16x8 a, f16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+// The tile loop of the head_dim-64 attention kernel without its bookkeeping.
+// PIPE false: per tile 8 score MFMAs, the softmax of the 32 scores of a lane, 8 P.V MFMAs.
+// PIPE true:  sixteen groups per tile, each one MFMA per 32-query block, the operand read for
+//             the group three groups on and an eighth of the softmax of a 32-key half:
+//             [S_b(t), PV_b(t-1)] under softmax(S_a(t)), then [PV_a(t), S_a(t+1)] under
+//             softmax(S_b(t)); nothing moves across a group's fence.
+// NQ: 32-query blocks per wavefront.  LOADS: each wavefront issues the product's four
+// global_load_lds per tile (K and V of a packed [512, 3, 384, 64] tensor, ring of three
+// stages) behind s_waitcnt vmcnt(4) and a block barrier.
+// stamps[2 * (4 * block + wave)] = shader clocks of the loop, [.. + 1] = constant-rate clocks.
+template <bool PIPE, int NQ, bool LOADS>
+__global__ __launch_bounds__(256, NQ == 1 ? 3 : 2) void probe_fmha_loop_kernel(float *__restrict__ sink,
+                                                                              uint64_t *__restrict__ stamps, int tiles,
+                                                                              float c, const char *__restrict__ kv) {
+  constexpr int kStageBytes = 16384, kStages = LOADS ? 3 : 2, AHEAD = 3;
+  constexpr uint32_t tokBytes = 3 * 384 * 128;
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[kStages * kStageBytes];
+  for (int i = threadIdx.x; i < kStages * kStageBytes / 4; i += 256)
+    reinterpret_cast<uint32_t *>(smem)[i] = 0x2e662e66u; // 0.1 in fp16
   __syncthreads();
-  const uint32_t lbase =
-      (uint32_t)(uintptr_t)((__attribute__((address_space(3))) unsigned char *)smem) + (threadIdx.x % 64) * 16;
-  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-  float a[8];
-  for (int i = 0; i < 8; i++) a[i] = 0.5f + 0.001f * (float)(threadIdx.x + i);
-  f16x8 ma, mb;
-  for (int i = 0; i < 8; i++) {
-    ma[i] = (_Float16)0.01f;
-    mb[i] = (_Float16)0.02f;
+  const int lane = threadIdx.x % 64, l32 = lane % 32, hl = lane / 32;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  const uint32_t ldsBase = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) unsigned char *)smem);
+  // operand addresses of the product kernel's head_dim-64 geometry (swizzled chunks)
+  uint32_t kfrag[4], vfrag[2];
+  for (int cc = 0; cc < 4; cc++) kfrag[cc] = (uint32_t)(l32 * 128 + (((2 * cc + hl) ^ ((l32 >> 1) & 7)) * 16));
+  {
+    const int g = lane / 16, L = lane % 16, r = L % 4, j = L / 4;
+    for (int db = 0; db < 2; db++) {
+      const int chunk = (4 * db + 2 * (g % 2) + r / 2) ^ ((((4 * hl + j) >> 1) & 1) << 2);
+      vfrag[db] = (uint32_t)((4 * hl + j) * 128 + chunk * 16 + 8 * (r % 2));
+    }
   }
-  f32x16 c0 = {}, c1 = {};
-  u32x4 ra = {0, 0, 0, 0};
-  u32x2 rb = {0, 0};
-  auto softmax8 = [&](int r) { // the softmax instructions of 8 scores
+  f16x8 qf[NQ][4];
+  for (int qi = 0; qi < NQ; qi++)
+    for (int cc = 0; cc < 4; cc++)
+      for (int i = 0; i < 8; i++) qf[qi][cc][i] = (_Float16)(0.01f * (float)((lane + cc + i + 3 * qi) % 7));
+  f32x16 accO[NQ][2] = {};
+  float l0[NQ] = {}, l1[NQ] = {};
+  const float mc = 0.25f * c;
+  const f32x16 zero = {};
+
+  auto kOp = [&](uint32_t stage, int half, int cc) -> f16x8 {
+    return *reinterpret_cast<const f16x8 __attribute__((address_space(3))) *>(
+        (const lds_u8 *)(uintptr_t)(ldsBase + stage + kfrag[cc]) + half * 32 * 128);
+  };
+  auto vOp = [&](uint32_t stage, int half, int db, int m) -> f16x8 {
+    const lds_u8 *p = (const lds_u8 *)(uintptr_t)(ldsBase + stage + 8192 + vfrag[db]) + (32 * half + 16 * m) * 128;
+    const f16x4 lo = probeReadTr(p), hi = probeReadTr(p + 8 * 128);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  struct SV { f32x16 v[NQ]; };
+  struct PV { f16x8 v[NQ][2]; };
+  auto scores = [&](uint32_t stage, int half) {
+    SV s;
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      asm volatile("v_fma_f32 %0, %0, %0, %0\n v_exp_f32 %0, %0\n v_add_f32 %1, %1, %0" : "+v"(a[i]), "+v"(a[(i + 1) & 7]));
-      if (i & 1) asm volatile("v_cvt_pk_f16_f32 %0, %0, %1" : "+v"(a[i]) : "v"(a[i - 1]));
-      if (MODE == 0) {
-        if (i == 0 || i == 4) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(ra) : "v"(lbase), "i"(r * 2048 + i * 128));
-        if (i & 1) {
-          asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(rb) : "v"(lbase), "i"(r * 2048 + i * 64));
-          if (i & 2) c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma, mb, c0, 0, 0, 0);
-          else c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma, mb, c1, 0, 0, 0);
-        }
+    for (int qi = 0; qi < NQ; qi++) s.v[qi] = zero;
+#pragma unroll
+    for (int cc = 0; cc < 4; cc++) {
+      const f16x8 a = kOp(stage, half, cc);
+#pragma unroll
+      for (int qi = 0; qi < NQ; qi++) s.v[qi] = probeMfma(a, qf[qi][cc], s.v[qi]);
+    }
+    return s;
+  };
+  auto pv = [&](uint32_t stage, int half, const PV &p) {
+#pragma unroll
+    for (int m = 0; m < 2; m++)
+#pragma unroll
+      for (int db = 0; db < 2; db++) {
+        const f16x8 a = vOp(stage, half, db, m);
+#pragma unroll
+        for (int qi = 0; qi < NQ; qi++) accO[qi][db] = probeMfma(a, p.v[qi][m], accO[qi][db]);
       }
+  };
+  // two scores of a 32-key half: fma, exp2, add, convert
+  auto chunk = [&](const f32x16 &sc, f16x8(&p)[2], float &a0, float &a1, int j) {
+    const float e0 = __builtin_amdgcn_exp2f(sc[2 * j] * c - mc), e1 = __builtin_amdgcn_exp2f(sc[2 * j + 1] * c - mc);
+    a0 += e0;
+    a1 += e1;
+    p[j / 4][(2 * j) % 8] = (_Float16)e0;
+    p[j / 4][(2 * j + 1) % 8] = (_Float16)e1;
+  };
+  auto softmax = [&](const SV &s, PV &p) {
+#pragma unroll
+    for (int qi = 0; qi < NQ; qi++)
+#pragma unroll
+      for (int j = 0; j < 8; j++) chunk(s.v[qi], p.v[qi], l0[qi], l1[qi], j);
+  };
+
+  // the product kernel's tile movers: 2 K loads + 2 V loads of 1 KiB per wavefront and tile
+  const int mrow = lane / 8, mchunk = lane % 8;
+  uint32_t koff[2], voff[2];
+  for (int i = 0; i < 2; i++) {
+    const int row = 8 * (2 * wave + i) + mrow;
+    koff[i] = (uint32_t)row * tokBytes + (uint32_t)((mchunk ^ ((row >> 1) & 7)) * 16);
+    voff[i] = (uint32_t)row * tokBytes + (uint32_t)((mchunk ^ (((row >> 1) & 1) << 2)) * 16);
+  }
+  const char *kbase = kv + (size_t)(blockIdx.x % 384) * 128 + 384 * 128; // the K column of one (batch, head)
+  const char *vbase = kbase + 384 * 128;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+  auto dma16 = [&](uint32_t voffset, const char *sbase, uint32_t ldsAddr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voffset), "s"(sbase), "s"(ldsAddr) : "memory", "m0");
+  };
+#pragma clang diagnostic pop
+  auto issueTile = [&](int kt) { // tiles 0..7 of the 512 tokens, over and over
+    const uint32_t kdst = ldsBase + (uint32_t)((kt % 3) * kStageBytes + (2 * wave) * 1024), vdst = kdst + 8192;
+    const char *kg = kbase + (size_t)(kt % 8) * 64 * tokBytes, *vg = vbase + (size_t)(kt % 8) * 64 * tokBytes;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      dma16(koff[i], kg, kdst + i * 1024);
+      dma16(voff[i], vg, vdst + i * 1024);
     }
   };
-  const uint64_t t0 = clock64();
-  for (int t = 0; t < tiles; t++) {
-    if (MODE == 1) {
-#pragma unroll
-      for (int r = 0; r < 8; r++) {
-        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(ra) : "v"(lbase), "i"(r * 1024));
-        if (r & 1) c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma, mb, c0, 0, 0, 0);
-        else c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma, mb, c1, 0, 0, 0);
-      }
-      a[0] += c0[0]; // the softmax starts from the scores
-      a[1] += c1[0];
+  auto stageOf = [&](int t) { return (uint32_t)(LOADS ? t % 3 : t & 1) * kStageBytes; };
+  auto arrive = [&](int t) { // tile t has landed for everybody; the stage of tile t - 1 is free for tile t + 2
+    if (LOADS) {
+      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      __syncthreads();
+      issueTile(t + 2);
     }
-#pragma unroll
-    for (int r = 0; r < 4; r++) softmax8(r);
-    if (MODE == 1) {
-      ma[0] = (_Float16)a[0]; // P.V starts from the softmax
-#pragma unroll
-      for (int r = 0; r < 8; r++) {
-        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(rb) : "v"(lbase), "i"(r * 1024));
-        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(rb) : "v"(lbase), "i"(r * 1024 + 512));
-        if (r & 1) c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma, mb, c0, 0, 0, 0);
-        else c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ma, mb, c1, 0, 0, 0);
-      }
-    }
+  };
+  if (LOADS) {
+    issueTile(0);
+    issueTile(1);
   }
-  asm volatile("s_waitcnt lgkmcnt(0)");
-  const uint64_t t1 = clock64();
-  float s = (float)(ra[0] + rb[0]);
-  for (int i = 0; i < 8; i++) s += a[i];
-  for (int i = 0; i < 16; i++) s += c0[i] + c1[i];
+  const uint64_t t0 = clock64(), w0 = wall_clock64();
+  if (!PIPE) {
+    for (int t = 0; t < tiles; t++) {
+      arrive(t);
+      const uint32_t stage = stageOf(t);
+      SV sa = scores(stage, 0), sb = scores(stage, 1);
+      PV pa, pb;
+      softmax(sa, pa);
+      softmax(sb, pb);
+      pv(stage, 0, pa);
+      pv(stage, 1, pb);
+    }
+  } else {
+    // Groups 0..7 of tile t: S_b(t) (4), PV_b(t-1) (4), under the softmax of S_a(t); groups 8..15:
+    // PV_a(t) (4), S_a(t+1) (4), under the softmax of S_b(t).  Tile t + 1 must have landed before
+    // group 12 - AHEAD reads its K operands: the barrier sits at group 8.
+    if (LOADS) {
+      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      __syncthreads();
+    }
+    SV sa = scores(stageOf(0), 0), sb;
+    PV pa = {}, pb = {};
+#pragma unroll
+    for (int qi = 0; qi < NQ; qi++) sb.v[qi] = zero;
+    f16x8 aop[16];
+    auto loadOp = [&](int g, uint32_t cur, uint32_t prev, uint32_t next) {
+      const int i = g % 8;
+      if (g < 8) aop[g] = i < 4 ? kOp(cur, 1, i) : vOp(prev, 1, (i - 4) % 2, (i - 4) / 2);
+      else aop[g] = i < 4 ? vOp(cur, 0, i % 2, i / 2) : kOp(next, 0, i - 4);
+    };
+#pragma unroll
+    for (int g = 0; g < AHEAD; g++) loadOp(g, stageOf(0), stageOf(0), stageOf(1));
+    for (int t = 0; t < tiles; t++) {
+      const uint32_t cur = stageOf(t), prev = stageOf(t + kStages - 1), next = stageOf(t + 1), next2 = stageOf(t + 2);
+#pragma unroll
+      for (int g = 0; g < 16; g++) {
+        if (g == 8 && LOADS) { // PV_b(t-1) is done: its stage takes tile t + 2; tile t + 1 has landed
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          __syncthreads();
+          issueTile(t + 2);
+        }
+        if (g + AHEAD < 16) loadOp(g + AHEAD, cur, prev, next);
+        else loadOp(g + AHEAD - 16, next, cur, next2);
+        const int i = g % 8;
+#pragma unroll
+        for (int qi = 0; qi < NQ; qi++) {
+          if (g < 8) {
+            if (i < 4) sb.v[qi] = probeMfma(aop[g], qf[qi][i], i == 0 ? zero : sb.v[qi]);
+            else accO[qi][(i - 4) % 2] = probeMfma(aop[g], pb.v[qi][(i - 4) / 2], accO[qi][(i - 4) % 2]);
+            chunk(sa.v[qi], pa.v[qi], l0[qi], l1[qi], i);
+          } else {
+            if (i < 4) accO[qi][i % 2] = probeMfma(aop[g], pa.v[qi][i / 2], accO[qi][i % 2]);
+            else sa.v[qi] = probeMfma(aop[g], qf[qi][i - 4], i == 4 ? zero : sa.v[qi]);
+            chunk(sb.v[qi], pb.v[qi], l0[qi], l1[qi], i);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    accO[0][0][0] += sa.v[0][0] + (float)pb.v[0][0][0] + sa.v[NQ - 1][1] + (float)pb.v[NQ - 1][1][1];
+  }
+  float s = 0.f;
+  for (int qi = 0; qi < NQ; qi++) {
+    s += l0[qi] + l1[qi];
+    for (int i = 0; i < 16; i++) s += accO[qi][0][i] + accO[qi][1][i];
+  }
+  if (LOADS) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  const uint64_t t1 = clock64(), w1 = wall_clock64();
   if (s == 12345.678f) sink[0] = s;
-  if (threadIdx.x == 0) stamps[blockIdx.x] = t1 - t0;
+  if (lane == 0) {
+    stamps[2 * (blockIdx.x * 4 + wave)] = t1 - t0;
+    stamps[2 * (blockIdx.x * 4 + wave) + 1] = w1 - w0;
+  }
 }
 
 template <typename F> float timed(F &&launch, int steps, int warmup, hipStream_t stream) {
@@ -177,24 +326,59 @@ float mgpuProbeMfma(void *sink, void *stamps, int blocks, int iters, uint64_t *s
   return ms;
 }
 
-// Mean shader clocks per tile and wavefront of the attention instruction mix (mode 0 interleaved,
-// 1 in phases) with `blocks` blocks of four wavefronts; stamps must hold `blocks` uint64.  < 0 on failure.
-double mgpuProbeFmhaMix(void *sink, void *stamps, int blocks, int tiles, int mode, void *stream) {
+// The attention tile-loop model (probe_fmha_loop_kernel) with `blocks` blocks of four wavefronts, `tiles`
+// tiles each.  variant: bit 0 = half-tile pipeline instead of phases, bit 1 = 64 instead of 32 queries per
+// wavefront, bit 2 = with the tile loads and the block barrier.  kv: a packed [512, 3, 384, 64] fp16 tensor
+// (75 497 472 bytes), read only with bit 2.  stamps must hold 8 * blocks uint64.  Returns the milliseconds
+// of the launch (< 0 on failure); *shaderClocks / *constClocks receive the mean clocks a wavefront spent in
+// the loop.
+float mgpuProbeFmhaLoop(void *sink, void *stamps, const void *kv, int blocks, int tiles, int variant,
+                        double *shaderClocks, double *constClocks, void *stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
-  for (int rep = 0; rep < 2; rep++) {
-    if (mode == 0) probe_fmha_mix_kernel<0><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<float *>(sink), static_cast<uint64_t *>(stamps), tiles);
-    else probe_fmha_mix_kernel<1><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<float *>(sink), static_cast<uint64_t *>(stamps), tiles);
-  }
-  if (hipStreamSynchronize(s) != hipSuccess || hipGetLastError() != hipSuccess) return -1.0;
-  uint64_t *host = new uint64_t[blocks];
-  double mean = -1.0;
-  if (hipMemcpy(host, stamps, sizeof(uint64_t) * blocks, hipMemcpyDeviceToHost) == hipSuccess) {
-    double total = 0.0;
-    for (int i = 0; i < blocks; i++) total += (double)host[i];
-    mean = total / blocks / tiles;
+  auto *sk = static_cast<float *>(sink);
+  auto *st = static_cast<uint64_t *>(stamps);
+  const auto *src = static_cast<const char *>(kv);
+  if ((variant & 4) && !src) return -1.0f;
+  const dim3 grid(blocks), block(256);
+  const float c = 0.18f;
+  const float ms = timed(
+      [&](int) {
+        switch (variant) {
+#define MGPU_PROBE_LOOP(V, PIPE, NQ, LOADS)                                                   \
+  case V:                                                                                     \
+    probe_fmha_loop_kernel<PIPE, NQ, LOADS><<<grid, block, 0, s>>>(sk, st, tiles, c, src);    \
+    break;
+          MGPU_PROBE_LOOP(0, false, 1, false)
+          MGPU_PROBE_LOOP(1, true, 1, false)
+          MGPU_PROBE_LOOP(2, false, 2, false)
+          MGPU_PROBE_LOOP(3, true, 2, false)
+          MGPU_PROBE_LOOP(4, false, 1, true)
+          MGPU_PROBE_LOOP(5, true, 1, true)
+          MGPU_PROBE_LOOP(6, false, 2, true)
+          MGPU_PROBE_LOOP(7, true, 2, true)
+#undef MGPU_PROBE_LOOP
+        default:
+          break;
+        }
+      },
+      1, 1, s);
+  if (ms < 0.0f) return ms;
+  const size_t n = (size_t)blocks * 4;
+  uint64_t *host = new uint64_t[2 * n];
+  float result = ms;
+  if (hipMemcpy(host, stamps, sizeof(uint64_t) * 2 * n, hipMemcpyDeviceToHost) == hipSuccess) {
+    double a = 0.0, b = 0.0;
+    for (size_t i = 0; i < n; i++) {
+      a += (double)host[2 * i];
+      b += (double)host[2 * i + 1];
+    }
+    *shaderClocks = a / (double)n;
+    *constClocks = b / (double)n;
+  } else {
+    result = -1.0f;
   }
   delete[] host;
-  return mean;
+  return result;
 }
 
 // Rate of the constant clock behind wall_clock64(), in kHz (0 if the runtime does not say).
