@@ -162,9 +162,11 @@ def test_bert_encoder_layer_config4(pkg, gpu, oracle):
         assert err.mean() <= 5e-4
 
 
-@pytest.mark.parametrize("causal,relu,d,H", [(True, True, 512, 8), (False, False, 512, 8), (True, True, 1024, 8)])
+@pytest.mark.parametrize("causal,relu,d,H", [(True, True, 512, 8), (False, False, 512, 8), (True, True, 1024, 8),
+                                             (True, False, 512, 2)])
 def test_decoding_context_layer(pkg, gpu, oracle, rng, causal, relu, d, H):
-    """(1024, 8): the reference's own head geometry, 8 heads of 128."""
+    """(1024, 8): the reference's own head geometry, 8 heads of 128; (512, 2): heads of 256, the widest of the
+    reference's attention kernel list."""
     B, S, ffn = 4, 128, 2048
     f = lambda *s, sc=0.03: (sc * rng.standard_normal(s)).astype(np.float32)
     x = rng.standard_normal((B, S, d)).astype(np.float32)
