@@ -592,20 +592,32 @@ void launch(const void *qkv, const int32_t *seqlens, const int32_t *cuSeqlens, v
   const auto *in = static_cast<const uint16_t *>(qkv);
   auto *o = static_cast<uint16_t *>(out);
   const dim3 grid((unsigned)blocks), block(256);
-  if (causal)
-    fmha_fwd_kernel<T, D, NQ, true, false, PAD><<<grid, block, 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, nullptr, dHead);
-  else
+  if (causal) {
+    // (the causal kernel exists with one 32-query block per wavefront only)
+    if constexpr (NQ == 1)
+      fmha_fwd_kernel<T, D, NQ, true, false, PAD><<<grid, block, 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, nullptr, dHead);
+    else
+      fail("fusedMHA: internal dispatch error");
+  } else {
     fmha_fwd_kernel<T, D, NQ, false, false, PAD><<<grid, block, 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, nullptr, dHead);
+  }
   MGPU_CHECK_LAUNCH("fmha_fwd_kernel");
 }
 
 template <typename T>
 void launchForHeadDim(const void *qkv, const int32_t *seqlens, const int32_t *cuSeqlens, void *out, int B, int S, int H,
                       int dHead, float scale, bool causal, hipStream_t stream) {
-  // One 32-query block per wavefront: 64 queries per wavefront would halve the
-  // LDS operand traffic per flop, but at 224 VGPRs only two wavefronts fit a
-  // SIMD and the kernel measured slower at every shape tried.
-  if (dHead == 64) launch<T, 64, 1, false>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
+  // One 32-query block per wavefront, except on long unmasked-or-padded sequences at
+  // head_dim 64: with 64 queries per wavefront every K / V operand read from LDS feeds
+  // two MFMAs and a block of 256 queries shares each tile load, which measured 3-10 %
+  // faster from S = 2048 on (b16 s2048 h12, b4 s4096 h16, b1 s16384 h8) - but at 229
+  // VGPRs only two wavefronts fit a SIMD, so the 256-query blocks must fill both block
+  // slots of every CU, and at S = 512 or 1024 prologue and epilogue of the fewer, larger
+  // blocks cost more than the loop gains (b32 s512 h12: 9 % slower).
+  const bool wideBlocks = dHead == 64 && !causal && S >= 2048 &&
+                          (int64_t)B * H * ((S + 255) / 256) >= 2 * (int64_t)deviceComputeUnits();
+  if (wideBlocks) launch<T, 64, 2, false>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
+  else if (dHead == 64) launch<T, 64, 1, false>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
   else if (dHead == 128) launch<T, 128, 1, false>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
   else if (dHead == 256) launch<T, 256, 1, false>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);
   else if (dHead < 64) launch<T, 64, 1, true>(qkv, seqlens, cuSeqlens, out, B, S, H, dHead, scale, causal, stream);

@@ -202,6 +202,32 @@ def test_fmha_identities_at_full_size(pkg, gpu):
     assert torch.equal(pkg.fused_mha(qkv), pkg.fused_mha(qkv))  # deterministic
 
 
+@pytest.mark.parametrize("B,S,H,ragged,dtype", [(8, 2048, 8, False, "f16"), (4, 2304, 16, True, "f16"),
+                                                 (8, 2048, 8, True, "bf16")])
+def test_fmha_long_sequences_with_64_queries_per_wavefront(pkg, gpu, oracle, B, S, H, ragged, dtype):
+    """From S = 2048 on, with enough (batch, head) pairs to give every CU two blocks of 256 queries, the
+    unmasked / key-padded head_dim-64 problem runs with 64 queries per wavefront (another instantiation of
+    the kernel): against the oracle with unit-variance operands, partial last query block (2304 = 9 x 256)
+    and ragged key counts included, and against the 32-query kernel, which the causal flag selects on a
+    problem whose mask hides nothing (key counts of 1: one admissible key per row either way)."""
+    import torch
+    rng = np.random.Generator(np.random.PCG64(S + H))
+    qkv = rng.standard_normal((B, S, 3, H, 64)).astype(np.float32)
+    lens = rng.integers(1, S + 1, B).astype(np.int32) if ragged else None
+    if ragged:
+        lens[0] = S
+    tq = torch.from_numpy(qkv).to(gpu).to(torch.float16 if dtype == "f16" else torch.bfloat16)
+    bits = tq.view(torch.int16).cpu().numpy().view(np.uint16)
+    tl = to_dev(lens, gpu) if ragged else None
+    got = pkg.fused_mha(tq, tl).float().cpu().numpy()
+    ref = oracle.fmha(bits.view(np.float16) if dtype == "f16" else bits, lens, bf16=dtype == "bf16")
+    assert excess(got, ref, TOL_F16 if dtype == "f16" else TOL_BF16) <= 1.0
+    one = to_dev(np.ones(B, np.int32), gpu)
+    a = pkg.fused_mha(tq, one).float()
+    b = pkg.fused_mha(tq, one, causal=True).float()
+    assert (a - b).abs().max().item() <= 1e-6
+
+
 def test_fmha_bf16(pkg, gpu, oracle, rng):
     import torch
     for (B, S, H, lens, causal) in [(2, 128, 2, None, False), (2, 200, 3, [200, 77], False), (1, 130, 1, None, True)]:
