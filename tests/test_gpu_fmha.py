@@ -228,6 +228,47 @@ def test_fmha_long_sequences_with_64_queries_per_wavefront(pkg, gpu, oracle, B, 
     assert (a - b).abs().max().item() <= 1e-6
 
 
+def test_fmha_seeded_shape_sweep(pkg, gpu, oracle):
+    """Forty problems drawn from a fixed seed over everything the entry points take: head sizes
+    8..256 (all three tile geometries and the sizes padded into them), S from 1 to a few tiles past
+    the block sizes, key counts with zeros and full lengths, causal or not, fp16 or bf16, padded
+    layout or packed rows behind prefix sums - each against the oracle."""
+    import torch
+    rng = np.random.Generator(np.random.PCG64(20260))
+    for case in range(40):
+        D = int(rng.choice([8, 16, 24, 32, 40, 48, 64, 72, 80, 96, 104, 128, 136, 144, 160, 192, 248, 256]))
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        S = int(rng.choice([1, 2, 31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 191, 200, 256, 257, 300, 385, 512, 640]))
+        causal = bool(rng.integers(0, 2))
+        bf16 = bool(rng.integers(0, 4) == 0)
+        mode = int(rng.integers(0, 3))  # 0: no lengths, 1: key counts, 2: packed rows with prefix sums
+        dt = torch.bfloat16 if bf16 else torch.float16
+        tol = TOL_BF16 if bf16 else TOL_F16
+        what = f"case {case}: D={D} B={B} H={H} S={S} causal={causal} bf16={bf16} mode={mode}"
+        if mode < 2:
+            lens = None
+            if mode == 1:
+                lens = rng.integers(0, S + 1, B).astype(np.int32)
+                lens[rng.integers(0, B)] = S
+            tq = torch.from_numpy(rng.standard_normal((B, S, 3, H, D)).astype(np.float32)).to(gpu).to(dt)
+            bits = tq.view(torch.int16).cpu().numpy().view(np.uint16)
+            got = pkg.fused_mha(tq, to_dev(lens, gpu) if lens is not None else None, causal=causal).float().cpu().numpy()
+            ref = oracle.fmha(bits if bf16 else bits.view(np.float16), lens, causal=causal, bf16=bf16)
+            assert excess(got, ref, tol) <= 1.0, what
+        else:
+            lens = rng.integers(0, S + 1, B)
+            lens[rng.integers(0, B)] = S
+            cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+            tq = torch.from_numpy(rng.standard_normal((int(cu[-1]), 3, H, D)).astype(np.float32)).to(gpu).to(dt)
+            got = pkg.fused_mha_cu_seqlens(tq, to_dev(cu, gpu), S, causal=causal).float().cpu().numpy()
+            bits = tq.view(torch.int16).cpu().numpy().view(np.uint16)
+            for b, n in enumerate(lens):
+                if n:
+                    rows = bits[cu[b]:cu[b + 1]][None]
+                    ref = oracle.fmha(rows if bf16 else rows.view(np.float16), causal=causal, bf16=bf16)[0]
+                    assert excess(got[cu[b]:cu[b + 1]], ref, tol) <= 1.0, what + f" sequence {b}"
+
+
 def test_fmha_bf16(pkg, gpu, oracle, rng):
     import torch
     for (B, S, H, lens, causal) in [(2, 128, 2, None, False), (2, 200, 3, [200, 77], False), (1, 130, 1, None, True)]:
