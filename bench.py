@@ -682,6 +682,13 @@ def main():
         fmha_case("fmha_d128_b4_s2048", "fused MHA fp16 b4 s2048 h32 d128 [long sequences, the reference layer's head size]",
                   4, 2048, 32, False, D=128)
 
+    if want("fmha_b4_s4096"):
+        fmha_case("fmha_b4_s4096", "fused MHA fp16 b4 s4096 h16 d64 [long sequences: 64 queries per wavefront]",
+                  4, 4096, 16, False)
+    if want("fmha_d256_b4_s2048"):
+        fmha_case("fmha_d256_b4_s2048", "fused MHA fp16 b4 s2048 h8 d256 [the widest head of the reference's kernel list]",
+                  4, 2048, 8, False, D=256)
+
     # ---------------- GEMM with fused epilogue ---------------------------------
     # The four GEMMs of the BERT-base layer at 4096 tokens.  mgpuMatmulExF16 runs whichever of the library (+ a
     # separate GELU pass where there is one) and the hand-written MFMA kernel the committed table names for the

@@ -48,6 +48,8 @@ ENTRIES = {
     "fmha_b32_s512_causal": (fmha(64, True), None, 100_663_296),
     "fmha_d128_b32_s512": (fmha(128, False), 32 * 8 * 4 * 256, 134_217_728),
     "fmha_d128_b4_s2048": (fmha(128, False), 4 * 32 * 16 * 256, 268_435_456),
+    "fmha_b4_s4096": (fmha(64, False), 4 * 16 * 16 * 256, 134_217_728),       # blocks of 256 queries
+    "fmha_d256_b4_s2048": (fmha(256, False), 4 * 8 * 16 * 256, 134_217_728),
 }
 COPY_KERNEL = r"copyBuffer"
 
