@@ -10,11 +10,11 @@
 //
 // Work decomposition.  A 256-thread block (4 wavefronts) owns BM = 128 * NQ
 // consecutive queries of one (batch, head); each wavefront owns NQ blocks of 32
-// queries.  Key/value tiles of 8 KiB (64 keys at head_dim 64, 32 keys at 128;
-// the comments below give the head_dim 64 numbers) travel HBM -> LDS directly
-// (global_load_lds, 16 bytes per lane, no register staging) into a ring of
-// three LDS stages shared by the 4 wavefronts, so two tiles are always in
-// flight behind the one being consumed.
+// queries.  Key/value tiles of 8 KiB (64 keys at head_dim 64; 16 KiB at 128 and
+// 256, see Geo below; the comments give the head_dim 64 numbers) travel HBM ->
+// LDS directly (global_load_lds, 16 bytes per lane, no register staging) into a
+// ring of three LDS stages shared by the 4 wavefronts, so two tiles are always
+// in flight behind the one being consumed.
 //
 // MFMA formulation (v_mfma_f32_32x32x16_{f16,bf16}; operand lane layout: lane l
 // supplies row/col l%32 and k-slots 8*(l/32)..+7; the 32x32 accumulator gives
@@ -75,21 +75,25 @@ namespace mgpu {
 
 namespace {
 
-// Geometry per head dimension D (64, 128 or 256).  A K or V tile is 8 KiB at 64 and
-// 128 - 64 keys of 128 bytes or 32 keys of 256 bytes, so both share the movers and
-// the MFMA count per tile (8 for the scores, 8 for P.V); at D = 128 a tile carries
-// half as many scores, i.e. half the softmax work per MFMA.  At D = 256 a tile is
-// 16 KiB (32 keys of 512 bytes, 16 + 16 MFMAs) and the ring has two stages, so that
-// two blocks still share a CU's LDS; their accumulators and Q operands (128 + 64
-// registers) leave room for two wavefronts per SIMD.
+// Geometry per head dimension D (64, 128 or 256).  At D = 64 a K or V tile is 8 KiB
+// (64 keys of 128 bytes, 8 MFMAs for the scores and 8 for P.V), the ring has three
+// stages and three blocks share a CU (146 VGPRs, three wavefronts per SIMD).  At
+// D = 128 and 256 a tile is 16 KiB (64 keys of 256 bytes or 32 of 512: 16 + 16 MFMAs
+// per tile, half as many barriers and bursts of tile loads per MFMA) and the ring has
+// two stages, so that two blocks share a CU's LDS; accumulators and Q operands (64 + 32
+// registers at 128, 128 + 64 at 256) leave room for two wavefronts per SIMD either way.
+// (D = 128 with 8 KiB tiles of 32 keys, a ring of three and three wavefronts per SIMD at
+// the 168-register limit measured 5-12 % slower from S = 128 to S = 8192 - b32 s512 h8
+// 50 against 44-51 us, b1 s8192 h8 273 against 257 - and 2 % faster only on the largest
+// grid tried, b4 s2048 h32.)
 template <int D> struct Geo {
   static_assert(D == 64 || D == 128 || D == 256, "head dimension 64, 128 or 256");
-  static constexpr int kTileBytes = D == 256 ? 16384 : 8192; // one K or V tile, unpadded rows
-  static constexpr int kStages = D == 256 ? 2 : 3;           // LDS ring depth
+  static constexpr int kTileBytes = D >= 128 ? 16384 : 8192; // one K or V tile, unpadded rows
+  static constexpr int kStages = D >= 128 ? 2 : 3;           // LDS ring depth
   static constexpr int kStageBytes = 2 * kTileBytes;         // a stage: the K tile followed by the V tile
-  static constexpr int LPW = kTileBytes / 4096;     // 1 KiB load instructions per wavefront and tile half: 2 / 2 / 4
-  static constexpr int kBN = kTileBytes / (D * 2);  // keys per tile: 64 / 32 / 32
-  static constexpr int KB = kBN / 32;               // 32-key score blocks per tile: 2 / 1 / 1
+  static constexpr int LPW = kTileBytes / 4096;     // 1 KiB load instructions per wavefront and tile half: 2 / 4 / 4
+  static constexpr int kBN = kTileBytes / (D * 2);  // keys per tile: 64 / 64 / 32
+  static constexpr int KB = kBN / 32;               // 32-key score blocks per tile: 2 / 2 / 1
   static constexpr int DC = D / 16;                 // MFMA k-steps over the head dimension: 4 / 8 / 16
   static constexpr int DB = D / 32;                 // 32-row blocks of O^T: 2 / 4 / 8
   static constexpr int rowBytes = D * 2;            // 128 / 256 / 512
