@@ -178,7 +178,7 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   // nQB - 1 - i are given to one work item, the long one first, so that every
   // work item carries the same number of tiles; left alone, the items with the
   // last query blocks run as long as without the mask while the others sit idle.
-  constexpr bool kCanPair = CAUSAL && D == 64; // elsewhere the second pass is compiled out
+  constexpr bool kCanPair = CAUSAL && D <= 128; // at 256 the second pass is compiled out
   const bool paired = kCanPair && pairItems;
   const int nItems = paired ? (nQB + 1) / 2 : nQB; // work items per (batch, head)
   const int item = wid % nItems;
@@ -587,9 +587,9 @@ void launch(const void *qkv, const int32_t *seqlens, const int32_t *cuSeqlens, v
   constexpr int BM = 128 * NQ;
   const int nQB = (S + BM - 1) / BM;
   // Causal query blocks go in pairs of equal total work when the head dimension
-  // is 64 (at 128 the second pass does not fit the register budget of three
+  // is 64 or 128 (at 256 the loop over the pair does not fit the registers of two
   // wavefronts per SIMD) and the halved grid still gives every CU two blocks.
-  const bool pair = causal && D == 64 && (int64_t)B * H * ((nQB + 1) / 2) >= 2 * (int64_t)deviceComputeUnits();
+  const bool pair = causal && D <= 128 && (int64_t)B * H * ((nQB + 1) / 2) >= 2 * (int64_t)deviceComputeUnits();
   const int64_t blocks = (int64_t)B * H * (pair ? (nQB + 1) / 2 : nQB);
   if (blocks > 0x7fffffffLL) fail("fusedMHA: problem too large for one launch");
   const float c = scale * 1.44269504088896340736f;
