@@ -395,6 +395,36 @@ def measure_ceilings(torch, loops, dev, gen, sp, ptrs, repeats) -> dict:
                                 "what": "v_mfma_f32_32x32x16_f16 on four independent accumulators from registers, "
                                         "4096 x 4 per wavefront, every SIMD of the device; shader clock from clock64() "
                                         "against the constant-rate wall_clock64()"}
+    # LDS read rate of the attention kernels' operand reads (csrc/tools/bench_probes.hip: probe_lds_read_kernel)
+    if hasattr(loops, "mgpuProbeLdsRead"):
+        loops.mgpuProbeLdsRead.restype = ctypes.c_float
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        lds_iters = 2000
+        lds_runs = []
+        for mode, name in ((0, "ds_read_b128"), (1, "ds_read_b64_tr_b16"), (2, "ds_read_b64")):
+            for waves_per_simd in (2, 3):
+                blocks = cus * waves_per_simd
+                best = None
+                for _ in range(3):
+                    sc, cc = ctypes.c_uint64(0), ctypes.c_uint64(0)
+                    ms = loops.mgpuProbeLdsRead(ctypes.c_void_p(sink.data_ptr()), ctypes.c_void_p(stamps.data_ptr()), blocks,
+                                                lds_iters, mode, ctypes.byref(sc), ctypes.byref(cc), sp)
+                    if ms > 0 and (best is None or ms < best[0]):
+                        best = (ms, sc.value, cc.value)
+                if best:
+                    ms, sc, cc = best
+                    nbytes = blocks * 4.0 * lds_iters * 16384
+                    ghz = sc / cc * khz / 1e6 if cc and khz else None
+                    lds_runs.append({"instruction": name, "wavefronts_per_simd": waves_per_simd,
+                                     "TB/s": round(nbytes / ms / 1e9, 1),
+                                     "shader_clock_ghz_in_kernel": ghz and round(ghz, 3),
+                                     "bytes_per_clock_and_cu": ghz and round(nbytes / ms / 1e6 / cus / ghz, 1)})
+        if lds_runs:
+            res["lds_read"] = {"runs": lds_runs,
+                               "what": "every wavefront re-reads a 16 KiB tile (64 rows of 256 bytes) 2000 times in the "
+                                       "operand patterns of the head_dim 128 attention tile: K operands by ds_read_b128, "
+                                       "V operands by the transposing ds_read_b64_tr_b16, and plain ds_read_b64; rate from "
+                                       "the launch's wall time, per clock with the shader clock read inside the kernel"}
     # the attention tile loop without its bookkeeping (csrc/tools/bench_probes.hip: probe_fmha_loop_kernel)
     kv = (torch.randn((512, 3, 384, 64), device=dev, generator=None) / 8).half()
     stamps = torch.zeros(8 * 256 * 3, dtype=torch.int64, device=dev)

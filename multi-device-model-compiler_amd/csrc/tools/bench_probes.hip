@@ -18,6 +18,11 @@
 //     barrier.  No masks, no row-maximum repair, no prologue or epilogue: what
 //     the SIMD, the LDS and the clock governor leave of the matrix rate for this
 //     mix, in shader clocks per tile and in wall-clock TFLOP/s.
+//   * the LDS read rate behind those operand reads: every wavefront of the
+//     device re-reads a 16 KiB tile (64 rows of 256 bytes, the head_dim 128
+//     geometry and its chunk swizzles) with ds_read_b128 in the K operand
+//     pattern, with ds_read_b64_tr_b16 in the V operand pattern, or with plain
+//     ds_read_b64.
 // Measurement plumbing only: nothing here is part of the kernel library.
 #include <hip/hip_runtime.h>
 
@@ -275,6 +280,73 @@ __global__ __launch_bounds__(256, NQ == 1 ? 3 : 2) void probe_fmha_loop_kernel(f
   }
 }
 
+// Every wavefront reads a 16 KiB tile `iters` times.  MODE 0: sixteen ds_read_b128, lane = (row
+// l % 32 [+32], 16-byte chunk (2c + l / 32) ^ (row & 15)) - the K operand reads of the head_dim 128
+// attention tile.  MODE 1: thirty-two ds_read_b64_tr_b16 in that tile's V operand pattern.
+// MODE 2: thirty-two ds_read_b64 of consecutive 8-byte pieces.
+// stamps[2 * block] = shader clocks, [2 * block + 1] = constant-rate clocks of wavefront 0.
+template <int MODE>
+__global__ __launch_bounds__(256) void probe_lds_read_kernel(uint32_t *__restrict__ sink, uint64_t *__restrict__ stamps,
+                                                              int iters) {
+  constexpr int rowBytes = 256;
+  __shared__ __attribute__((aligned(1024))) unsigned char tile[16384];
+  const int tid = threadIdx.x, lane = tid % 64, l32 = lane % 32, hl = lane / 32;
+  for (int i = tid; i < 16384 / 4; i += 256) reinterpret_cast<uint32_t *>(tile)[i] = (uint32_t)i * 2654435761u;
+  __syncthreads();
+  const uint32_t base = (uint32_t)(uintptr_t)((lds_u8 *)tile);
+  uint32_t kf[8], vf[4];
+  for (int c = 0; c < 8; c++) kf[c] = base + l32 * rowBytes + (((2 * c + hl) ^ (l32 & 15)) * 16);
+  for (int db = 0; db < 4; db++) {
+    const int g = lane / 16, L = lane % 16, r = L % 4, row = 4 * hl + L / 4;
+    vf[db] = base + row * rowBytes + (((4 * db + 2 * (g % 2) + r / 2) ^ ((row & 3) << 2)) * 16) + 8 * (r % 2);
+  }
+  // The reads are written as assembly so that nothing but the read itself is issued per
+  // operand: the results go nowhere, one s_waitcnt per tile collects them.
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  u32x4 wide = {0u, 0u, 0u, 0u};
+  u32x2 narrow = {0u, 0u};
+  const uint64_t t0 = clock64(), w0 = wall_clock64();
+  for (int it = 0; it < iters; it++) {
+    if (MODE == 0) {
+#pragma unroll
+      for (int c = 0; c < 8; c++) {
+        asm volatile("ds_read_b128 %0, %1" : "=v"(wide) : "v"(kf[c]));
+        asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(wide) : "v"(kf[c]));
+      }
+    } else if (MODE == 1) {
+#pragma unroll
+      for (int db = 0; db < 4; db++) { // keys 8 * k8 + 4 * hl + 0..3, k8 = 0..7
+        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(narrow) : "v"(vf[db]));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:2048" : "=v"(narrow) : "v"(vf[db]));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:4096" : "=v"(narrow) : "v"(vf[db]));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:6144" : "=v"(narrow) : "v"(vf[db]));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:8192" : "=v"(narrow) : "v"(vf[db]));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:10240" : "=v"(narrow) : "v"(vf[db]));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:12288" : "=v"(narrow) : "v"(vf[db]));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:14336" : "=v"(narrow) : "v"(vf[db]));
+      }
+    } else {
+      const uint32_t lin = base + lane * 8;
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const uint32_t at = lin + i * 2048;
+        asm volatile("ds_read_b64 %0, %1" : "=v"(narrow) : "v"(at));
+        asm volatile("ds_read_b64 %0, %1 offset:512" : "=v"(narrow) : "v"(at));
+        asm volatile("ds_read_b64 %0, %1 offset:1024" : "=v"(narrow) : "v"(at));
+        asm volatile("ds_read_b64 %0, %1 offset:1536" : "=v"(narrow) : "v"(at));
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+  const uint64_t t1 = clock64(), w1 = wall_clock64();
+  u32x4 acc = {wide[0] ^ narrow[0], wide[1] ^ narrow[1], wide[2], wide[3]};
+  if (acc[0] == 0x12345u && acc[1] == 7u) sink[0] = acc[2] ^ acc[3]; // keeps the reads alive
+  if (threadIdx.x == 0) {
+    stamps[2 * blockIdx.x] = t1 - t0;
+    stamps[2 * blockIdx.x + 1] = w1 - w0;
+  }
+}
+
 template <typename F> float timed(F &&launch, int steps, int warmup, hipStream_t stream) {
   for (int i = 0; i < warmup; i++) launch(i);
   if (hipStreamSynchronize(stream) != hipSuccess) return -1.0f;
@@ -382,6 +454,30 @@ float mgpuProbeFmhaLoop(void *sink, void *stamps, const void *kv, int blocks, in
 }
 
 // Rate of the constant clock behind wall_clock64(), in kHz (0 if the runtime does not say).
+// probe_lds_read_kernel: one launch of `blocks` blocks of four wavefronts, each wavefront reading 16 KiB of
+// LDS `iters` times.  mode 0 = ds_read_b128 (K operand pattern), 1 = ds_read_b64_tr_b16 (V operand pattern),
+// 2 = ds_read_b64.  Returns the milliseconds of the launch (< 0 on failure); *shaderClocks / *constClocks
+// receive the clocks wavefront 0 of block 0 spent in its loop; stamps must hold 2 * blocks uint64.
+float mgpuProbeLdsRead(void *sink, void *stamps, int blocks, int iters, int mode, uint64_t *shaderClocks,
+                       uint64_t *constClocks, void *stream) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto *sk = static_cast<uint32_t *>(sink);
+  auto *st = static_cast<uint64_t *>(stamps);
+  if (mode < 0 || mode > 2 || blocks <= 0 || iters <= 0) return -1.0f;
+  const float ms = timed(
+      [&](int) {
+        if (mode == 0) probe_lds_read_kernel<0><<<dim3(blocks), dim3(256), 0, s>>>(sk, st, iters);
+        else if (mode == 1) probe_lds_read_kernel<1><<<dim3(blocks), dim3(256), 0, s>>>(sk, st, iters);
+        else probe_lds_read_kernel<2><<<dim3(blocks), dim3(256), 0, s>>>(sk, st, iters);
+      },
+      1, 1, s);
+  uint64_t host[2] = {0, 0};
+  if (hipMemcpy(host, stamps, sizeof(host), hipMemcpyDeviceToHost) != hipSuccess) return -1.0f;
+  *shaderClocks = host[0];
+  *constClocks = host[1];
+  return ms;
+}
+
 int mgpuProbeWallClockKHz(void) {
   int dev = 0, khz = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
