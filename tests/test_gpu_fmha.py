@@ -85,6 +85,54 @@ def test_fmha_causal(pkg, gpu, oracle, rng, B, S, H, lens):
     assert excess(got, oracle.fmha(qkv, lens, causal=True), TOL_F16) <= 1.0
 
 
+@pytest.mark.parametrize("D,B,S,H,ragged,dtype", [
+    (64, 32, 512, 12, False, "f16"),   # four query blocks per (batch, head): pairs (3, 0) and (2, 1)
+    (64, 16, 640, 16, True, "f16"),    # five: pairs (4, 0), (3, 1) and block 2 alone; ragged key counts
+    (128, 32, 512, 8, False, "f16"),   # the 128-wide geometry, exactly two work items per CU
+    (128, 16, 384, 16, True, "bf16"),  # three query blocks: pair (2, 0) and block 1 alone
+    (40, 32, 512, 12, True, "f16"),    # a head size padded into the 64-wide geometry
+])
+def test_fmha_causal_paired_query_blocks(pkg, gpu, oracle, D, B, S, H, ragged, dtype):
+    """On grids that leave every CU two work items afterwards (batch x heads x ceil(query blocks / 2) >= 2 x CUs),
+    the causal kernel gives query block i and block nQB - 1 - i to one work item, which runs them one after the
+    other through the same LDS ring; the small problems of the other causal tests never get there."""
+    import torch
+    nqb = (S + 127) // 128
+    assert B * H * ((nqb + 1) // 2) >= 2 * torch.cuda.get_device_properties(gpu).multi_processor_count
+    rng = np.random.Generator(np.random.PCG64(D * 1000 + S))
+    tq = torch.from_numpy(rng.standard_normal((B, S, 3, H, D)).astype(np.float32)).to(gpu)
+    tq = tq.to(torch.float16 if dtype == "f16" else torch.bfloat16)
+    bits = tq.view(torch.int16).cpu().numpy().view(np.uint16)
+    lens = None
+    if ragged:
+        lens = rng.integers(0, S + 1, B).astype(np.int32)
+        lens[0], lens[1] = S, 1
+    got = pkg.fused_mha(tq, to_dev(lens, gpu) if ragged else None, causal=True).float().cpu().numpy()
+    ref = oracle.fmha(bits.view(np.float16) if dtype == "f16" else bits, lens, causal=True, bf16=dtype == "bf16")
+    assert excess(got, ref, TOL_F16 if dtype == "f16" else TOL_BF16) <= 1.0
+
+
+def test_fmha_causal_paired_query_blocks_over_packed_rows(pkg, gpu, oracle):
+    """The same pairing with the sequences given as prefix sums over packed rows: a pair's late block may lie
+    wholly beyond a short sequence while its early block does not."""
+    import torch
+    B, S, H, D = 40, 512, 8, 64
+    rng = np.random.Generator(np.random.PCG64(4051))
+    lens = rng.integers(0, S + 1, B)
+    lens[:6] = [S, 0, 1, 128, 129, 385]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    tq = torch.from_numpy(rng.standard_normal((int(cu[-1]), 3, H, D)).astype(np.float32)).to(gpu).half()
+    guard = torch.full((int(cu[-1]) + 64, H * D), 7.0, device=gpu, dtype=torch.float16)
+    pkg.fused_mha_cu_seqlens(tq, to_dev(cu, gpu), S, causal=True, out=guard[:int(cu[-1])])
+    assert (guard[int(cu[-1]):] == 7.0).all()  # nothing written past the last row
+    got = guard[:int(cu[-1])].float().cpu().numpy()
+    bits = tq.view(torch.int16).cpu().numpy().view(np.uint16)
+    for b, n in enumerate(lens):
+        if n:
+            ref = oracle.fmha(bits[cu[b]:cu[b + 1]][None].view(np.float16), causal=True)[0]
+            assert excess(got[cu[b]:cu[b + 1]], ref, TOL_F16) <= 1.0, f"sequence {b} of {n} rows"
+
+
 def test_fmha_large_logits_and_other_scales(pkg, gpu, oracle, rng):
     """Peaked softmax rows: the kernel produces P against a stale reference
     maximum and repairs overflow after the fact, so rows whose scores keep
@@ -284,7 +332,7 @@ def test_fmha_bf16(pkg, gpu, oracle, rng):
 @pytest.mark.parametrize("lens,max_s,causal,D,dtype", [
     ([128, 128, 128], 128, False, 64, "f16"),          # the dense call written as prefix sums
     ([5, 0, 300, 64, 1, 129], 300, False, 64, "f16"),  # ragged, an empty sequence, tile boundaries
-    ([200, 77, 512], 512, True, 64, "f16"),            # causal: paired query blocks over packed rows
+    ([200, 77, 512], 512, True, 64, "f16"),            # causal over packed rows
     ([33, 250], 256, False, 128, "f16"),
     ([100, 260], 260, True, 64, "bf16"),
 ])
@@ -341,7 +389,7 @@ def test_fmha_profile_entry_point_matches_the_product_kernel(pkg, gpu):
 @pytest.mark.parametrize("D,B,S,H,lens,causal,dtype", [
     (32, 2, 200, 3, None, False, "f16"),       # the reference's kernel list holds 32, 40, 80 next to 64 and 128
     (40, 2, 257, 2, [257, 90], False, "f16"),
-    (40, 1, 384, 2, None, True, "f16"),         # causal, paired query blocks in the 64-wide geometry
+    (40, 1, 384, 2, None, True, "f16"),         # causal in the 64-wide geometry
     (80, 2, 130, 3, [130, 1], False, "f16"),
     (80, 1, 300, 2, None, True, "bf16"),
     (96, 2, 96, 2, None, False, "bf16"),
