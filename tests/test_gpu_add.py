@@ -76,6 +76,36 @@ def test_add_large_and_properties(pkg, gpu, rng):
     assert torch.equal(c.view(torch.int32), exact.view(torch.int32))
 
 
+def test_add_beyond_the_grid_cap(pkg, gpu):
+    """The launch is capped at 2^22 blocks; beyond 2^32 + 1024 elements on the vector path (2^30 on the scalar
+    path, which unaligned pointers take) a block walks on by the size of the grid.  Checked on the device against
+    the fp64 sum rounded once, a slice at a time; 52 GB of device memory."""
+    import torch
+    n = (1 << 32) + 4 * 256 * 3 + 7
+    if torch.cuda.mem_get_info(gpu)[0] < 60 * (1 << 30):
+        pytest.skip("needs 60 GB of free device memory")
+    a = torch.empty(n, device=gpu).uniform_(-1e3, 1e3)
+    b = torch.empty(n, device=gpu).uniform_(-1.0, 1.0)
+    c = torch.zeros(n + 8, device=gpu)
+
+    def same(lo, hi, shift=0):
+        step = 1 << 28
+        for i in range(lo, hi, step):
+            j = min(hi, i + step)
+            exact = (a[i:j].double() + b[i:j].double()).float()
+            if not torch.equal(c[i + shift:j + shift].view(torch.int32), exact.view(torch.int32)):
+                return False
+        return True
+
+    pkg.add(a, b, out=c[:n])
+    assert same(0, n) and c[n:].abs().sum().item() == 0
+    # the scalar path: every pointer one element off 16-byte alignment
+    m = (1 << 30) + 5
+    c.zero_()
+    pkg.add(a[1:1 + m], b[1:1 + m], out=c[1:1 + m])
+    assert same(1, 1 + m) and c[0].item() == 0 and c[1 + m:1 + m + 1024].abs().sum().item() == 0
+
+
 def test_add_empty(pkg, gpu):
     import torch
     e = torch.empty(0, device=gpu)

@@ -22,9 +22,10 @@ def spacing_tol(ref, mant_bits, floor):
 
 
 # M, K, N.  The launcher picks 128- or 96-column tiles and a reduction step of 32 or 64 from the shape (on the 256
-# CUs of the test device): both widths and both steps are in the list, N = 672 and 96 only divide by 96.
+# CUs of the test device): both widths and both steps are in the list, N = 672 and 96 only divide by 96, and
+# (8192, 128, 672) is 448 tiles of 96 columns with the input rows fetched for two steps at a time.
 SHAPES = [(128, 32, 128), (128, 64, 256), (256, 96, 384), (384, 160, 128), (256, 1024, 128), (256, 64, 96),
-          (128, 32, 672), (512, 768, 768), (1024, 768, 3072), (4096, 768, 2304), (4096, 64, 3072)]
+          (128, 32, 672), (512, 768, 768), (1024, 768, 3072), (4096, 768, 2304), (4096, 64, 3072), (8192, 128, 672)]
 
 
 def epilogues(pkg, oracle, tb, b, tr, r):
