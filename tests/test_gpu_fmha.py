@@ -276,6 +276,27 @@ def test_fmha_long_sequences_with_64_queries_per_wavefront(pkg, gpu, oracle, B, 
     assert (a - b).abs().max().item() <= 1e-6
 
 
+def test_fmha_long_packed_rows_with_64_queries_per_wavefront(pkg, gpu, oracle):
+    """The 64-query instantiation behind the prefix-sum entry point: sequences of up to 2048 packed rows, among them
+    an empty one, one of a single row, and lengths either side of the 256-query block size."""
+    import torch
+    B, S, H = 8, 2048, 8
+    rng = np.random.Generator(np.random.PCG64(77))
+    lens = np.array([S, 0, 1, 255, 256, 257, 1300, 2047])
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    total = int(cu[-1])
+    tq = torch.from_numpy(rng.standard_normal((total, 3, H, 64)).astype(np.float32)).to(gpu).half()
+    guard = torch.full((total + 64, H * 64), 7.0, device=gpu, dtype=torch.float16)
+    pkg.fused_mha_cu_seqlens(tq, to_dev(cu, gpu), S, out=guard[:total])
+    assert (guard[total:] == 7.0).all()
+    got = guard[:total].float().cpu().numpy()
+    bits = tq.view(torch.int16).cpu().numpy().view(np.uint16)
+    for b, n in enumerate(lens):
+        if n:
+            ref = oracle.fmha(bits[cu[b]:cu[b + 1]][None].view(np.float16))[0]
+            assert excess(got[cu[b]:cu[b + 1]], ref, TOL_F16) <= 1.0, f"sequence {b} of {n} rows"
+
+
 def test_fmha_seeded_shape_sweep(pkg, gpu, oracle):
     """Forty problems drawn from a fixed seed over everything the entry points take: head sizes
     8..256 (all three tile geometries and the sizes padded into them), S from 1 to a few tiles past
