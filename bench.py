@@ -368,6 +368,14 @@ def measure_ceilings(torch, loops, dev, gen, sp, ptrs, repeats) -> dict:
             "cache_resident_us_per_launch": round(warm * 10, 3),
             "what": "the same copy kernel at the headline's byte count (12.6 MB in, 12.6 MB out, 3072 blocks): the time "
                     "a launch of that size costs a kernel that does nothing but move the bytes"}
+        # the same sets, half of each: the byte count of the fp16 LayerNorm configuration
+        quarter = half // 2
+        cold16 = med(lambda: loops.mgpuProbeCopy(ptrs(srcs), ptrs(dsts), nsets, ctypes.c_size_t(quarter), 100, 10, sp))
+        if cold16:
+            res["copy_at_fp16_layernorm_size"] = {
+                "bytes": 2 * quarter, "us_per_launch": round(cold16 * 10, 3),
+                "GB/s": round(2 * quarter * 100 / cold16 / 1e6, 1),
+                "what": "the copy kernel at the byte count of LayerNorm fp16 (32,128,768): 6.3 MB in, 6.3 MB out"}
     del srcs, dsts
     sink = torch.zeros(16, device=dev)
     stamps = torch.zeros(2 * 4096, dtype=torch.int64, device=dev)
