@@ -18,11 +18,14 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 // (3,640,640) shape: plain loads + non-temporal stores with one vector per lane
 // and one block per 256 vectors is the fastest combination (non-temporal LOADS
 // cost about 10 %, more vectors per lane do not help at this size).
+//
+// Everything the kernel needs arrives as an explicit argument (the grid's stride included,
+// instead of gridDim): the explicit arguments are preloaded into SGPRs, the grid dimensions
+// would cost a load from the kernarg segment on the path to the first data load.
 template <int UNROLL>
 __global__ __launch_bounds__(256) void add_f32_vec4_kernel(const float4v *__restrict__ a,
                                                            const float4v *__restrict__ b,
-                                                           float4v *__restrict__ c, int64_t n4) {
-  const int64_t stride = (int64_t)gridDim.x * 256 * UNROLL;
+                                                           float4v *__restrict__ c, int64_t n4, int64_t stride) {
   for (int64_t base = (int64_t)blockIdx.x * 256 * UNROLL + threadIdx.x; base < n4; base += stride) {
     float4v va[UNROLL], vb[UNROLL];
 #pragma unroll
@@ -64,7 +67,7 @@ void addF32(const float *a, const float *b, float *c, int64_t n, hipStream_t str
     if (blocks > cap) blocks = cap;
     add_f32_vec4_kernel<UNROLL><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
         reinterpret_cast<const float4v *>(a), reinterpret_cast<const float4v *>(b),
-        reinterpret_cast<float4v *>(c), n4);
+        reinterpret_cast<float4v *>(c), n4, blocks * 256 * UNROLL);
     MGPU_CHECK_LAUNCH("add_f32_vec4_kernel");
     if (n % 4) {
       add_f32_scalar_kernel<<<dim3(1), dim3(64), 0, stream>>>(a, b, c, n4 * 4, n);

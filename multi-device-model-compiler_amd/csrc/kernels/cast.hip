@@ -19,10 +19,12 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 // T is the 16-bit type (_Float16 or bf16_t); its vectors travel as 16 raw bytes.
+// (The grid's stride is an explicit argument: explicit arguments are preloaded into SGPRs,
+// gridDim would be a load from the kernarg segment in front of the first data load.)
 template <typename T>
 __global__ __launch_bounds__(256) void cast_f32_to_h_vec8_kernel(u32x4 *__restrict__ dst,
-                                                                 const f32x4 *__restrict__ src, size_t n8) {
-  const size_t stride = (size_t)gridDim.x * 256;
+                                                                 const f32x4 *__restrict__ src, size_t n8,
+                                                                 size_t stride) {
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += stride) {
     const f32x4 lo = src[2 * i];
     const f32x4 hi = src[2 * i + 1];
@@ -33,8 +35,8 @@ __global__ __launch_bounds__(256) void cast_f32_to_h_vec8_kernel(u32x4 *__restri
 
 template <typename T>
 __global__ __launch_bounds__(256) void cast_h_to_f32_vec8_kernel(f32x4 *__restrict__ dst,
-                                                                 const u32x4 *__restrict__ src, size_t n8) {
-  const size_t stride = (size_t)gridDim.x * 256;
+                                                                 const u32x4 *__restrict__ src, size_t n8,
+                                                                 size_t stride) {
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += stride) {
     float v[8];
     ElemTraits<T>::unpack(src[i], v);
@@ -114,8 +116,9 @@ void castFromF32(void *dst, const float *src, size_t size, hipStream_t stream, c
   size_t done = 0;
   if (aligned16(dst) && aligned16(src) && size >= 8) {
     const size_t n8 = size / 8;
-    cast_f32_to_h_vec8_kernel<T><<<dim3(gridFor(n8, 256)), dim3(256), 0, stream>>>(
-        reinterpret_cast<u32x4 *>(d), reinterpret_cast<const f32x4 *>(src), n8);
+    const unsigned blocks = gridFor(n8, 256);
+    cast_f32_to_h_vec8_kernel<T><<<dim3(blocks), dim3(256), 0, stream>>>(
+        reinterpret_cast<u32x4 *>(d), reinterpret_cast<const f32x4 *>(src), n8, (size_t)blocks * 256);
     MGPU_CHECK_LAUNCH("cast_f32_to_h_vec8_kernel");
     done = n8 * 8;
   }
@@ -133,8 +136,9 @@ void castToF32(float *dst, const void *src, size_t size, hipStream_t stream, con
   size_t done = 0;
   if (aligned16(dst) && aligned16(src) && size >= 8) {
     const size_t n8 = size / 8;
-    cast_h_to_f32_vec8_kernel<T><<<dim3(gridFor(n8, 256)), dim3(256), 0, stream>>>(
-        reinterpret_cast<f32x4 *>(dst), reinterpret_cast<const u32x4 *>(s), n8);
+    const unsigned blocks = gridFor(n8, 256);
+    cast_h_to_f32_vec8_kernel<T><<<dim3(blocks), dim3(256), 0, stream>>>(
+        reinterpret_cast<f32x4 *>(dst), reinterpret_cast<const u32x4 *>(s), n8, (size_t)blocks * 256);
     MGPU_CHECK_LAUNCH("cast_h_to_f32_vec8_kernel");
     done = n8 * 8;
   }

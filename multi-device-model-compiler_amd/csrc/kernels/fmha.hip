@@ -142,7 +142,10 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
                                                               const int32_t *__restrict__ cuSeqlens,
                                                               uint16_t *__restrict__ out, int S, int H,
                                                               int nQB, float scale_log2e, int pairItems,
-                                                              uint64_t *__restrict__ stamps, int dHead) {
+                                                              int nblk, int dHead,
+                                                              uint64_t *__restrict__ stamps) {
+  // (nblk is the grid size: as an explicit argument it is one of the fourteen dwords the
+  // command processor preloads into SGPRs; gridDim would be a load from the kernarg segment)
   uint64_t tEntry = 0, wEntry = 0, tFirstTile = 0, tLoopEnd = 0;
   uint64_t cWait = 0, cScores = 0, cSoftmax = 0, cPV = 0, tMark = 0;
   if (TRACE) {
@@ -170,7 +173,6 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   // contiguous run of work items goes to each of the 8 XCDs (consecutive block
   // ids are dealt round-robin to the XCDs), so the blocks that re-read the
   // same K/V share one L2.
-  const int nblk = gridDim.x;
   const int bid = blockIdx.x;
   const int wid = (nblk % 8 == 0) ? (bid % 8) * (nblk / 8) + bid / 8 : bid;
   // Causal: query block i of a (batch, head) needs i + 1 of the nQB key
@@ -612,11 +614,11 @@ void launch(const void *qkv, const int32_t *seqlens, const int32_t *cuSeqlens, v
   if (causal) {
     // (the causal kernel exists with one 32-query block per wavefront only)
     if constexpr (NQ == 1)
-      fmha_fwd_kernel<T, D, NQ, true, false, PAD><<<grid, block, 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, nullptr, dHead);
+      fmha_fwd_kernel<T, D, NQ, true, false, PAD><<<grid, block, 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, (int)blocks, dHead, nullptr);
     else
       fail("fusedMHA: internal dispatch error");
   } else {
-    fmha_fwd_kernel<T, D, NQ, false, false, PAD><<<grid, block, 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, nullptr, dHead);
+    fmha_fwd_kernel<T, D, NQ, false, false, PAD><<<grid, block, 0, stream>>>(in, seqlens, cuSeqlens, o, S, H, nQB, c, pair ? 1 : 0, (int)blocks, dHead, nullptr);
   }
   MGPU_CHECK_LAUNCH("fmha_fwd_kernel");
 }
@@ -679,7 +681,7 @@ int64_t fusedMHAProfile(const void *qkv, void *out, int B, int S, int H, float s
   if (blocks > 0x7fffffffLL) fail("fusedMHAProfile: problem too large for one launch");
   fmha_fwd_kernel<_Float16, 64, 1, false, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
       static_cast<const uint16_t *>(qkv), nullptr, nullptr, static_cast<uint16_t *>(out), S, H, nQB,
-      scale * 1.44269504088896340736f, 0, stamps, 64);
+      scale * 1.44269504088896340736f, 0, (int)blocks, 64, stamps);
   MGPU_CHECK_LAUNCH("fmha_fwd_kernel (profile)");
   return blocks;
 }

@@ -74,7 +74,7 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256, BK == 32 ? 3 : 1) void gemm_mfma
                                                                         const uint16_t *__restrict__ weight,
                                                                         const uint16_t *__restrict__ bias,
                                                                         const uint16_t *residual, uint16_t *out, int N,
-                                                                        int K, int tilesN) {
+                                                                        int K, int tilesN, int tilesM) {
   using M = Mma<T>;
   using v8 = typename M::v8;
   using v4 = typename M::v4;
@@ -107,10 +107,11 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256, BK == 32 ? 3 : 1) void gemm_mfma
   // slices they load per step are then few (8 input + 12 weight slices instead
   // of 2 + 64 for a row-major sweep of a wide matrix) and hit in that XCD's L2.
   constexpr int kGroup = 8;
-  const int nblk = gridDim.x;
+  // (the grid is tilesM x tilesN blocks; both are explicit arguments - fourteen dwords in all,
+  // what the command processor preloads into SGPRs - rather than gridDim, a kernarg-segment load)
+  const int nblk = tilesM * tilesN;
   const int bid = blockIdx.x;
   const int wid = (nblk % 8 == 0) ? (bid % 8) * (nblk / 8) + bid / 8 : bid;
-  const int tilesM = nblk / tilesN;
   const int perGroup = kGroup * tilesN;
   const int firstM = (wid / perGroup) * kGroup;
   const int groupRows = tilesM - firstM < kGroup ? tilesM - firstM : kGroup;
@@ -419,11 +420,11 @@ void launchTile(const uint16_t *a, const uint16_t *w, const uint16_t *b, const u
   const int tilesN = (int)(N / (32 * NB));
   const dim3 grid((unsigned)((M / kBM) * tilesN)), block(SPLIT ? 512 : 256);
   if (act == ACT_GELU)
-    gemm_mfma_kernel<T, ACT_GELU, BK, NB, PAIRED, SPLIT><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+    gemm_mfma_kernel<T, ACT_GELU, BK, NB, PAIRED, SPLIT><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN, (int)(M / kBM));
   else if (act == ACT_RELU)
-    gemm_mfma_kernel<T, ACT_RELU, BK, NB, PAIRED, SPLIT><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+    gemm_mfma_kernel<T, ACT_RELU, BK, NB, PAIRED, SPLIT><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN, (int)(M / kBM));
   else
-    gemm_mfma_kernel<T, ACT_NONE, BK, NB, PAIRED, SPLIT><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN);
+    gemm_mfma_kernel<T, ACT_NONE, BK, NB, PAIRED, SPLIT><<<grid, block, 0, stream>>>(a, w, b, r, o, (int)N, (int)K, tilesN, (int)(M / kBM));
 }
 
 // Tile width: the one under which the busiest CU carries the fewest columns

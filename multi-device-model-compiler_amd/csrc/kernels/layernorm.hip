@@ -28,12 +28,16 @@ constexpr int kMaxVPL = 8; // vectors per lane the register kernel is built for
 // it the branches that would sit between the loads).
 template <typename T, int LANES, int VPL, bool RESIDUAL, bool FULL>
 __global__ __launch_bounds__(256) void layernorm_rows_kernel(
-    const T *__restrict__ input, const T *__restrict__ residual, const T *__restrict__ gamma,
-    const T *__restrict__ beta, T *__restrict__ sumOut, T *__restrict__ normed, float eps, int m,
-    int n) {
+    const T *__restrict__ input, const T *__restrict__ gamma, const T *__restrict__ beta, T *__restrict__ normed,
+    int m, int nArg, int rowStep, float eps, const T *__restrict__ residual, T *__restrict__ sumOut) {
+  // Argument order: the first 14 dwords are preloaded into SGPRs, and what the path to the
+  // first row load needs comes first; rowStep (rows per trip of the grid) stands in for
+  // gridDim, which would be a load from the kernarg segment.  A FULL row has a length the
+  // instantiation knows.
   using Tr = ElemTraits<T>;
   constexpr int VEC = Tr::kVec; // elements per 16-byte vector
   constexpr int GROUPS = 256 / LANES;
+  const int n = FULL ? LANES * VPL * VEC : nArg;
   const int lane = threadIdx.x % LANES;
   const int group = threadIdx.x / LANES;
   const int nvec = n / VEC;
@@ -55,7 +59,7 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
     }
   }
 
-  for (int row = blockIdx.x * GROUPS + group; row < m; row += gridDim.x * GROUPS) {
+  for (int row = blockIdx.x * GROUPS + group; row < m; row += rowStep) {
     const u32x4 *xv = reinterpret_cast<const u32x4 *>(input + (size_t)row * n);
     const u32x4 *rv = RESIDUAL ? reinterpret_cast<const u32x4 *>(residual + (size_t)row * n) : nullptr;
 
@@ -143,10 +147,12 @@ template <typename T, int LANES, int VPL, bool FULL>
 __global__ __launch_bounds__(256) void layernorm_cast_rows_kernel(const float *__restrict__ input,
                                                                   const T *__restrict__ gamma,
                                                                   const T *__restrict__ beta, T *__restrict__ castOut,
-                                                                  T *__restrict__ normed, float eps, int m, int n) {
+                                                                  T *__restrict__ normed, int m, int nArg, int rowStep,
+                                                                  float eps) {
   using Tr = ElemTraits<T>;
   constexpr int VEC = Tr::kVec; // 8
   constexpr int GROUPS = 256 / LANES;
+  const int n = FULL ? LANES * VPL * VEC : nArg; // (arguments: as in layernorm_rows_kernel)
   const int lane = threadIdx.x % LANES;
   const int group = threadIdx.x / LANES;
   const int nvec = n / VEC;
@@ -164,7 +170,7 @@ __global__ __launch_bounds__(256) void layernorm_cast_rows_kernel(const float *_
     }
   }
 
-  for (int row = blockIdx.x * GROUPS + group; row < m; row += gridDim.x * GROUPS) {
+  for (int row = blockIdx.x * GROUPS + group; row < m; row += rowStep) {
     const u32x4 *xv = reinterpret_cast<const u32x4 *>(input + (size_t)row * n);
     u32x4 lo[VPL], hi[VPL];
 #pragma unroll
@@ -239,11 +245,11 @@ __global__ __launch_bounds__(256) void layernorm_cast_rows_kernel(const float *_
 // and the barriers per row and keeps more loads in flight.
 template <typename T, int VPL, int ROWS, bool RESIDUAL, bool FULL>
 __global__ __launch_bounds__(256) void layernorm_block_kernel(
-    const T *__restrict__ input, const T *__restrict__ residual, const T *__restrict__ gamma,
-    const T *__restrict__ beta, T *__restrict__ sumOut, T *__restrict__ normed, float eps, int m,
-    int n) {
+    const T *__restrict__ input, const T *__restrict__ gamma, const T *__restrict__ beta, T *__restrict__ normed,
+    int m, int nArg, int rowStep, float eps, const T *__restrict__ residual, T *__restrict__ sumOut) {
   using Tr = ElemTraits<T>;
   constexpr int VEC = Tr::kVec;
+  const int n = FULL ? 256 * VPL * VEC : nArg; // (arguments: as in layernorm_rows_kernel)
   __shared__ float partial[2][ROWS][4];
   const int t = threadIdx.x, wave = t / 64;
   const int nvec = n / VEC;
@@ -251,7 +257,7 @@ __global__ __launch_bounds__(256) void layernorm_block_kernel(
   const u32x4 *gv = reinterpret_cast<const u32x4 *>(gamma);
   const u32x4 *bv = reinterpret_cast<const u32x4 *>(beta);
 
-  for (int row0 = blockIdx.x * ROWS; row0 < m; row0 += gridDim.x * ROWS) {
+  for (int row0 = blockIdx.x * ROWS; row0 < m; row0 += rowStep) {
     float x[ROWS][VPL][VEC];
     float sum[ROWS];
     {
@@ -361,14 +367,13 @@ __global__ __launch_bounds__(256) void layernorm_block_kernel(
 // row (the second and third hit in cache).
 template <typename T, bool RESIDUAL>
 __global__ __launch_bounds__(256) void layernorm_general_kernel(
-    const T *__restrict__ input, const T *__restrict__ residual, const T *__restrict__ gamma,
-    const T *__restrict__ beta, T *__restrict__ sumOut, T *__restrict__ normed, float eps, int m,
-    int n) {
+    const T *__restrict__ input, const T *__restrict__ gamma, const T *__restrict__ beta, T *__restrict__ normed,
+    int m, int n, int rowStep, float eps, const T *__restrict__ residual, T *__restrict__ sumOut) {
   using Tr = ElemTraits<T>;
   __shared__ float partial[4];
   const int wave = threadIdx.x / 64;
   const float inv_n = 1.0f / (float)n;
-  for (int row = blockIdx.x; row < m; row += gridDim.x) {
+  for (int row = blockIdx.x; row < m; row += rowStep) {
     const T *xr = input + (size_t)row * n;
     const T *rr = RESIDUAL ? residual + (size_t)row * n : nullptr;
     auto value = [&](int i) {
@@ -416,10 +421,10 @@ void launchRows(const T *input, const T *residual, const T *gamma, const T *beta
   if (blocks > cap) blocks = cap;
   if (n / ElemTraits<T>::kVec == LANES * VPL)
     layernorm_rows_kernel<T, LANES, VPL, RESIDUAL, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
-        input, residual, gamma, beta, sumOut, normed, eps, m, n);
+        input, gamma, beta, normed, m, n, (int)(blocks * GROUPS), eps, residual, sumOut);
   else
     layernorm_rows_kernel<T, LANES, VPL, RESIDUAL, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
-        input, residual, gamma, beta, sumOut, normed, eps, m, n);
+        input, gamma, beta, normed, m, n, (int)(blocks * GROUPS), eps, residual, sumOut);
   MGPU_CHECK_LAUNCH("layernorm_rows_kernel");
 }
 
@@ -480,7 +485,7 @@ void layerNormTyped(const T *input, const T *residual, const T *gamma, const T *
     if (pairRows) blocks = (blocks + 1) / 2;
 #define MGPU_LN_BLOCK(V, R, F)                                                                    \
   layernorm_block_kernel<T, V, R, RESIDUAL, F><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>( \
-      input, residual, gamma, beta, sumOut, normed, eps, m, n)
+      input, gamma, beta, normed, m, n, (int)(blocks * R), eps, residual, sumOut)
     if (vpl == 4 && pairRows) {
       if (full) MGPU_LN_BLOCK(4, 2, true); else MGPU_LN_BLOCK(4, 2, false);
     } else if (vpl == 4) {
@@ -499,7 +504,7 @@ void layerNormTyped(const T *input, const T *residual, const T *gamma, const T *
     return;
   }
   layernorm_general_kernel<T, RESIDUAL><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
-      input, residual, gamma, beta, sumOut, normed, eps, m, n);
+      input, gamma, beta, normed, m, n, (int)blocks, eps, residual, sumOut);
   MGPU_CHECK_LAUNCH("layernorm_general_kernel");
 }
 
@@ -562,10 +567,10 @@ bool castLayerNormF32ToF16(const float *input, const void *gamma, const void *be
   if (lanes == L && vpl == V) {                                                                                \
     if (full)                                                                                                  \
       layernorm_cast_rows_kernel<_Float16, L, V, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(      \
-          input, g, b, c, y, eps, m, n);                                                                       \
+          input, g, b, c, y, m, n, (int)(blocks * (256 / L)), eps);                                            \
     else                                                                                                       \
       layernorm_cast_rows_kernel<_Float16, L, V, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(     \
-          input, g, b, c, y, eps, m, n);                                                                       \
+          input, g, b, c, y, m, n, (int)(blocks * (256 / L)), eps);                                            \
   }
   MGPU_LN_CAST(16, 1) MGPU_LN_CAST(16, 2) MGPU_LN_CAST(16, 3) MGPU_LN_CAST(16, 4)
   MGPU_LN_CAST(32, 3) MGPU_LN_CAST(32, 4)
