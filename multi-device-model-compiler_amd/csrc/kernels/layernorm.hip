@@ -43,13 +43,29 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
   const int nvec = n / VEC;
   const float inv_n = 1.0f / (float)n;
 
-  // gamma and beta do not depend on the row: fetch them once, ahead of the row
-  // data, so that their latency is not paid between the reductions and the
-  // stores (a wavefront usually owns a single row and its run time is one
-  // chain of latencies).
+  // gamma and beta do not depend on the row: fetch them once, at the top, so that
+  // their latency is not paid between the reductions and the stores (a wavefront
+  // usually owns a single row and its run time is one chain of latencies) - but
+  // behind the loads of the first row: loads return in order, and the row is what
+  // the chain waits for first (fp32 (4096, 768): 4.46 -> 4.27 us).
   const u32x4 *gv = reinterpret_cast<const u32x4 *>(gamma);
   const u32x4 *bv = reinterpret_cast<const u32x4 *>(beta);
   u32x4 graw[VPL], braw[VPL];
+  u32x4 raw[VPL], rawr[VPL];
+  auto loadRow = [&](int row) {
+    const u32x4 *xv = reinterpret_cast<const u32x4 *>(input + (size_t)row * n);
+    const u32x4 *rv = RESIDUAL ? reinterpret_cast<const u32x4 *>(residual + (size_t)row * n) : nullptr;
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = lane + k * LANES;
+      if (FULL || v < nvec) {
+        raw[k] = xv[v];
+        if (RESIDUAL) rawr[k] = rv[v];
+      }
+    }
+  };
+  const int row0 = blockIdx.x * GROUPS + group;
+  if (row0 < m) loadRow(row0);
 #pragma unroll
   for (int k = 0; k < VPL; k++) {
     const int v = lane + k * LANES;
@@ -59,19 +75,8 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
     }
   }
 
-  for (int row = blockIdx.x * GROUPS + group; row < m; row += rowStep) {
-    const u32x4 *xv = reinterpret_cast<const u32x4 *>(input + (size_t)row * n);
-    const u32x4 *rv = RESIDUAL ? reinterpret_cast<const u32x4 *>(residual + (size_t)row * n) : nullptr;
-
-    u32x4 raw[VPL], rawr[VPL];
-#pragma unroll
-    for (int k = 0; k < VPL; k++) {
-      const int v = lane + k * LANES;
-      if (FULL || v < nvec) {
-        raw[k] = xv[v];
-        if (RESIDUAL) rawr[k] = rv[v];
-      }
-    }
+  for (int row = row0; row < m; row += rowStep) {
+    if (row != row0) loadRow(row);
 
     float x[VPL][VEC];
     float sum = 0.0f;
@@ -161,6 +166,21 @@ __global__ __launch_bounds__(256) void layernorm_cast_rows_kernel(const float *_
   const u32x4 *gv = reinterpret_cast<const u32x4 *>(gamma);
   const u32x4 *bv = reinterpret_cast<const u32x4 *>(beta);
   u32x4 graw[VPL], braw[VPL];
+  u32x4 lo[VPL], hi[VPL];
+  auto loadRow = [&](int row) {
+    const u32x4 *xv = reinterpret_cast<const u32x4 *>(input + (size_t)row * n);
+#pragma unroll
+    for (int k = 0; k < VPL; k++) {
+      const int v = lane + k * LANES;
+      if (FULL || v < nvec) {
+        lo[k] = xv[2 * v];
+        hi[k] = xv[2 * v + 1];
+      }
+    }
+  };
+  // (the first row's loads go out ahead of gamma and beta, as in layernorm_rows_kernel)
+  const int row0 = blockIdx.x * GROUPS + group;
+  if (row0 < m) loadRow(row0);
 #pragma unroll
   for (int k = 0; k < VPL; k++) {
     const int v = lane + k * LANES;
@@ -170,17 +190,8 @@ __global__ __launch_bounds__(256) void layernorm_cast_rows_kernel(const float *_
     }
   }
 
-  for (int row = blockIdx.x * GROUPS + group; row < m; row += rowStep) {
-    const u32x4 *xv = reinterpret_cast<const u32x4 *>(input + (size_t)row * n);
-    u32x4 lo[VPL], hi[VPL];
-#pragma unroll
-    for (int k = 0; k < VPL; k++) {
-      const int v = lane + k * LANES;
-      if (FULL || v < nvec) {
-        lo[k] = xv[2 * v];
-        hi[k] = xv[2 * v + 1];
-      }
-    }
+  for (int row = row0; row < m; row += rowStep) {
+    if (row != row0) loadRow(row);
 
     u32x4 *cv = reinterpret_cast<u32x4 *>(castOut + (size_t)row * n);
     float x[VPL][VEC];
