@@ -24,6 +24,8 @@
 //     pattern, with ds_read_b64_tr_b16 in the V operand pattern, or with plain
 //     ds_read_b64.
 // Measurement plumbing only: nothing here is part of the kernel library.
+#include "bench_timed.hpp"
+
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -38,6 +40,13 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(const u32x4 *__restrict
                                                           size_t vectors) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i < vectors) __builtin_nontemporal_store(src[i], dst + i);
+}
+
+// Two streams in, one out: the memory pattern of the elementwise add (the XOR stands in for the add).
+__global__ __launch_bounds__(256) void probe_combine_kernel(const u32x4 *__restrict__ a, const u32x4 *__restrict__ b,
+                                                             u32x4 *__restrict__ dst, size_t vectors) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < vectors) __builtin_nontemporal_store(a[i] ^ b[i], dst + i);
 }
 
 // iters x 4 MFMAs per wavefront; stamps[2 * block] = shader clocks, [2 * block + 1] = constant-rate clocks
@@ -347,20 +356,7 @@ __global__ __launch_bounds__(256) void probe_lds_read_kernel(uint32_t *__restric
   }
 }
 
-template <typename F> float timed(F &&launch, int steps, int warmup, hipStream_t stream) {
-  for (int i = 0; i < warmup; i++) launch(i);
-  if (hipStreamSynchronize(stream) != hipSuccess) return -1.0f;
-  hipEvent_t e0, e1;
-  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return -1.0f;
-  (void)hipEventRecord(e0, stream);
-  for (int i = 0; i < steps; i++) launch(i);
-  (void)hipEventRecord(e1, stream);
-  float ms = -1.0f;
-  if (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&ms, e0, e1) != hipSuccess) ms = -1.0f;
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
-  return hipGetLastError() == hipSuccess ? ms : -1.0f;
-}
+using mgpu_bench::timed;
 
 } // namespace
 
@@ -372,9 +368,25 @@ float mgpuProbeCopy(void *const *src, void *const *dst, int nsets, size_t bytes,
   const unsigned blocks = (unsigned)((vectors + 255) / 256);
   hipStream_t s = static_cast<hipStream_t>(stream);
   return timed(
-      [&](int i) {
+      [&](unsigned long i) {
         probe_copy_kernel<<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const u32x4 *>(src[i % nsets]),
                                                              static_cast<u32x4 *>(dst[i % nsets]), vectors);
+      },
+      steps, warmup, s);
+}
+
+// Milliseconds for `steps` launches that read `bytes` from a[i % nsets] and from b[i % nsets] and write
+// `bytes` to dst[i % nsets].
+float mgpuProbeCombine(void *const *a, void *const *b, void *const *dst, int nsets, size_t bytes, int steps, int warmup,
+                       void *stream) {
+  const size_t vectors = bytes / 16;
+  const unsigned blocks = (unsigned)((vectors + 255) / 256);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return timed(
+      [&](unsigned long i) {
+        probe_combine_kernel<<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const u32x4 *>(a[i % nsets]),
+                                                                static_cast<const u32x4 *>(b[i % nsets]),
+                                                                static_cast<u32x4 *>(dst[i % nsets]), vectors);
       },
       steps, warmup, s);
 }
@@ -386,7 +398,7 @@ float mgpuProbeMfma(void *sink, void *stamps, int blocks, int iters, uint64_t *s
                     void *stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float ms = timed(
-      [&](int) {
+      [&](unsigned long) {
         probe_mfma_kernel<<<dim3(blocks), dim3(256), 0, s>>>(static_cast<float *>(sink), static_cast<uint64_t *>(stamps),
                                                             iters);
       },
@@ -414,7 +426,7 @@ float mgpuProbeFmhaLoop(void *sink, void *stamps, const void *kv, int blocks, in
   const dim3 grid(blocks), block(256);
   const float c = 0.18f;
   const float ms = timed(
-      [&](int) {
+      [&](unsigned long) {
         switch (variant) {
 #define MGPU_PROBE_LOOP(V, PIPE, NQ, LOADS)                                                   \
   case V:                                                                                     \
@@ -465,7 +477,7 @@ float mgpuProbeLdsRead(void *sink, void *stamps, int blocks, int iters, int mode
   auto *st = static_cast<uint64_t *>(stamps);
   if (mode < 0 || mode > 2 || blocks <= 0 || iters <= 0) return -1.0f;
   const float ms = timed(
-      [&](int) {
+      [&](unsigned long) {
         if (mode == 0) probe_lds_read_kernel<0><<<dim3(blocks), dim3(256), 0, s>>>(sk, st, iters);
         else if (mode == 1) probe_lds_read_kernel<1><<<dim3(blocks), dim3(256), 0, s>>>(sk, st, iters);
         else probe_lds_read_kernel<2><<<dim3(blocks), dim3(256), 0, s>>>(sk, st, iters);
