@@ -79,7 +79,7 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the copy / launch-floor / MFMA-loop probes")
     ap.add_argument("--tune-gemm", action="store_true",
-                    help="measure the four GEMM shapes of the BERT-base layer with mgpuMatmulExTune (library candidates "
+                    help="measure the four GEMM shapes of the BERT-base layer with the tuner of the launch-loop library (library candidates "
                          "against the hand-written kernel) and print the lines of csrc/kernels/gemm_table.inc on stderr")
     ap.add_argument("--fmha-phases", action="store_true",
                     help="also run the attention kernel's profiling entry point at b32 s512 h12 d64 and report where a "
@@ -290,7 +290,7 @@ def cpu_baselines(pkg, m, n, ln_bytes) -> dict:
 
 
 def fmha_phases(torch, lib, loops, dev, gen, B=32, S=512, H=12) -> dict:
-    """Per-block clock stamps of the attention kernel (mgpuFusedMHAF16Profile):
+    """Per-block clock stamps of the attention kernel (mgpuBenchFusedMHAF16Profile of the launch-loop library):
     how long a block spends before its first tile, per tile, and after its last
     tile, and how the blocks fill the launch."""
     D = 64
@@ -300,10 +300,10 @@ def fmha_phases(torch, lib, loops, dev, gen, B=32, S=512, H=12) -> dict:
     stamps = torch.zeros(nblocks * 10, dtype=torch.int64, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     for _ in range(3):
-        got = lib.mgpuFusedMHAF16Profile(qkv.data_ptr(), out.data_ptr(), B, S, H, D ** -0.5, stamps.data_ptr(), stream)
+        got = loops.mgpuBenchFusedMHAF16Profile(qkv.data_ptr(), out.data_ptr(), B, S, H, D ** -0.5, stamps.data_ptr(), stream)
     torch.cuda.synchronize()
     if got != nblocks:
-        raise RuntimeError("mgpuFusedMHAF16Profile failed")
+        raise RuntimeError("mgpuBenchFusedMHAF16Profile failed")
     t = stamps.cpu().numpy().reshape(nblocks, 10).astype(np.float64)
     khz = int(loops.mgpuProbeWallClockKHz()) if loops else 100000
     wall_us = lambda ticks: ticks / khz * 1e3
@@ -405,7 +405,6 @@ def measure_ceilings(torch, loops, dev, gen, sp, ptrs, repeats) -> dict:
                                         "against the constant-rate wall_clock64()"}
     # LDS read rate of the attention kernels' operand reads (csrc/tools/bench_probes.hip: probe_lds_read_kernel)
     if hasattr(loops, "mgpuProbeLdsRead"):
-        loops.mgpuProbeLdsRead.restype = ctypes.c_float
         cus = torch.cuda.get_device_properties(dev).multi_processor_count
         lds_iters = 2000
         lds_runs = []
@@ -499,11 +498,7 @@ def main():
         # K calls of the C-ABI entry point from a C++ loop between two events on
         # the launch stream (lib/libmgpu_bench_loops.so): the call rate of a
         # compiled model, which a Python caller cannot reach
-        loops = ctypes.CDLL(os.path.join(pkg.LIB_DIR, "libmgpu_bench_loops.so"))
-        for fn in ("mgpuBenchLayerNormF32", "mgpuBenchLayerNormF16", "mgpuBenchAddF32", "mgpuBenchFusedMHAF16",
-                   "mgpuBenchBertEncoderLayerF16", "mgpuProbeCopy", "mgpuProbeMfma"):
-            getattr(loops, fn).restype = ctypes.c_float
-        loops.mgpuProbeFmhaLoop.restype = ctypes.c_float
+        loops = pkg.bench_loops()
     bench_stream = torch.cuda.Stream()
 
     def ptrs(tensors):
@@ -736,7 +731,7 @@ def main():
     # The four GEMMs of the BERT-base layer at 4096 tokens.  mgpuMatmulExF16 runs whichever of the library (+ a
     # separate GELU pass where there is one) and the hand-written MFMA kernel the committed table names for the
     # shape; mgpuGemmMfmaF16 is the hand-written kernel by itself.  With --tune-gemm the shape is first measured
-    # on this device (mgpuMatmulExTune) and the table line that measurement gives is printed.
+    # on this device (mgpuBenchTuneMatmulEx of the launch-loop library) and the table line that measurement gives is printed.
     def gemm_case(name, workload, M_, K_, N_, act, residual):
         x = torch.randn((M_, K_), device=dev, generator=gen).half()
         wt = (0.02 * torch.randn((K_, N_), device=dev, generator=gen)).half()
@@ -757,9 +752,13 @@ def main():
 
         tuned = None
         if args.tune_gemm:
-            tuned = int(lib.mgpuMatmulExTune(1, M_, N_, K_, 1, act, int(residual)))
-            check()
-            print(f"{{1, {M_}, {N_}, {K_}, 1, {act}, {int(residual)}, {tuned}}},", file=sys.stderr)
+            lib_us, mfma_us = ctypes.c_float(0), ctypes.c_float(0)
+            tuned = int(pkg.bench_loops().mgpuBenchTuneMatmulEx(1, M_, N_, K_, 1, act, int(residual),
+                                                                ctypes.byref(lib_us), ctypes.byref(mfma_us)))
+            if tuned < 0:
+                raise RuntimeError("mgpuBenchTuneMatmulEx failed")
+            print(f"{{1, {M_}, {N_}, {K_}, 1, {act}, {int(residual)}, {tuned}}},  // library {lib_us.value:.1f} us, "
+                  f"hand-written {mfma_us.value:.1f} us", file=sys.stderr)
         us_auto, us_mfma = gemm(lib.mgpuMatmulExF16), gemm(lib.mgpuGemmMfmaF16)
         flop = 2.0 * M_ * N_ * K_
         kernels.append({"name": name, "workload": workload,
@@ -885,7 +884,7 @@ def main():
     if loops and not args.no_ceilings:
         ceilings = measure_ceilings(torch, loops, dev, gen, sp, ptrs, R)
 
-    phases = fmha_phases(torch, lib, loops, dev, gen) if args.fmha_phases else None
+    phases = fmha_phases(torch, lib, pkg.bench_loops(), dev, gen) if args.fmha_phases else None
 
     # ---------------- CPU baseline: the CPU op library on the host cores --------
     cpu = None

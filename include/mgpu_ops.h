@@ -118,26 +118,17 @@ void mgpuFusedMHABF16(const void *qkv, const int32_t *seqlens, void *out, int32_
  * cu_seqlens holds B + 1 int32 prefix sums over token rows packed back to back,
  * qkv is [total, 3, H, D] and out [total, H*D] with total = cu_seqlens[B];
  * sequence b owns rows cu_seqlens[b] .. cu_seqlens[b+1]-1, attends only inside
- * itself, and max_s bounds the longest sequence (longer ones are cut to max_s
- * keys and rows).  With cu_seqlens = {0, S, 2S, ...} this is the dense call. */
+ * itself, and max_s bounds the longest sequence: the grid is sized by it, so a
+ * sequence longer than max_s is cut to its first max_s keys and ITS OUTPUT ROWS
+ * BEYOND max_s ARE NOT WRITTEN (the lengths live in device memory; the call
+ * does not wait to read them, so it cannot reject such a sequence - pass the
+ * true maximum).  With cu_seqlens = {0, S, 2S, ...} this is the dense call. */
 void mgpuFusedMHAF16CuSeqlens(const void *qkv, const int32_t *cu_seqlens, void *out, int32_t B,
                               int32_t max_s, int32_t H, int32_t D, float scale, int32_t causal,
                               mgpuStream_t stream);
 void mgpuFusedMHABF16CuSeqlens(const void *qkv, const int32_t *cu_seqlens, void *out, int32_t B,
                                int32_t max_s, int32_t H, int32_t D, float scale, int32_t causal,
                                mgpuStream_t stream);
-
-/* Profiling aid, no counterpart in the reference: mgpuFusedMHAF16 for head_dim
- * 64 without masks, with the kernel's own clocks recorded per 256-thread block.
- * stamps receives ten uint64 per block (device memory, 10 * return value
- * entries; blocks = B * H * ceil(S / 128)), all from wavefront 0 of the block:
- * the shader clock at block entry, when the first K/V tile has landed, after
- * the last tile, after the output stores were issued; the device-wide
- * constant-rate clock at entry and exit; and the shader clocks, summed over the
- * block's tiles, spent waiting for a tile to land, in the score MFMAs, in the
- * softmax and in the P.V MFMAs.  Returns the number of blocks (0 on error). */
-int64_t mgpuFusedMHAF16Profile(const void *qkv, void *out, int32_t B, int32_t S, int32_t H, float scale,
-                               uint64_t *stamps, mgpuStream_t stream);
 
 /* ---- casts (Utils.h:6-8; lib/Kernels/GPU/Utils.cu:85-103) ------------- */
 void mgpuCastF32ToF16(void *dst, const float *src, size_t size, mgpuStream_t stream);
@@ -193,15 +184,11 @@ void mgpuMatmulExBF16(void *input, void *weight, void *bias, void *output, void 
 
 /* mgpuMatmulEx* only enqueue: which kernel serves a shape (the library's or the
  * hand-written MFMA kernel below) comes from a table decided offline and a
- * fixed rule.  A caller who wants a shape measured on its own device asks for
- * it here, once, OUTSIDE any stream capture: the call allocates scratch
- * operands, times the library's candidates and the hand-written kernel
- * (synchronous, tens of milliseconds) and keeps the winner for the rest of the
- * process.  dtype: 0 fp32, 1 fp16, 2 bf16.  Returns 1 when the hand-written
- * kernel was kept, 0 for the library, -1 on error.  No counterpart in the
- * reference (it takes cuBLASLt's first heuristic, Ops.cu:186-200). */
-int32_t mgpuMatmulExTune(int32_t dtype, int64_t M, int64_t N, int64_t K, int32_t hasBias,
-                         int32_t hasRelu, int32_t hasResidual);
+ * fixed rule, never from a measurement inside this library; MGPU_GEMM_KERNEL =
+ * library | mfma in the environment overrides both.  The first library GEMM on
+ * a stream allocates that stream's 32 MiB workspace (hipMalloc, outside stream
+ * capture; a stream first seen under capture runs an algorithm that needs no
+ * workspace). */
 
 /* The hand-written MFMA kernel that serves mgpuMatmulExF16 / BF16 where it is
  * the faster path, callable by itself (no counterpart in the reference):
@@ -215,8 +202,12 @@ void mgpuGemmMfmaBF16(void *input, void *weight, void *bias, void *output, void 
                       int32_t hasResidual, mgpuStream_t stream);
 
 /* ---- transformer layers ----------------------------------------------- */
-/* Pre-LN layer, fp32 in/out, fp16 compute; same signature as the reference
- * (Ops.h:43-48; lib/Kernels/GPU/LLM.cu:26-159). */
+/* Transformer layer, fp32 in/out, fp16 compute; same signature as the reference
+ * (Ops.h:43-48; lib/Kernels/GPU/LLM.cu:26-159).  norm_first = true is the reference's
+ * pre-LN dataflow, y = x + proj(attention(LN(x))), out = y + ffn(LN(y)); norm_first =
+ * false (declared but never read by the reference's bodies) is the post-LN ordering of
+ * the same blocks, h = LN(x + proj(attention(x))), out = LN(h + ffn(h)).  Both
+ * LayerNorms have gamma = 1, beta = 0, eps = 1e-5, as in the reference. */
 void mgpuLLMDecodingContextLayer(float *input, float *qkv, float *gemm_weight, float *gemm_bias,
                                  float *ffn1_weight, float *ffn1_bias, float *ffn2_weight,
                                  float *ffn2_bias, float *output, int64_t batch, int64_t seq_len,
@@ -250,6 +241,8 @@ void mgpuBertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, 
  *   must fit in 48 MiB (BERT-base (32,128,768), ffn 3072: 36 MiB);
  *   batch*seq_len a multiple of 128, d_model and feed_forward_dim multiples
  *   of 128 (or 96) and of 32, operands 16-byte aligned.
+ * A rejected call enqueues nothing.  The stream must belong to the device that
+ * is current when the call is made (the array's address is that device's).
  * Every call on one GPU shares that GPU's array: calls that overlap in time on
  * different streams of one GPU race; calls on one stream are ordered. */
 void mgpuBertEncoderLayerF16NoAlloc(const void *x, const void *wqkv, const void *bqkv, const void *wo,

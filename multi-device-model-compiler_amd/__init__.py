@@ -59,7 +59,6 @@ OPS_SIGNATURES = {
     "mgpuFusedMHABF16": (None, [_c_void_p] * 3 + [_c_int32] * 4 + [_c_float, _c_int32, _c_void_p]),
     "mgpuFusedMHAF16CuSeqlens": (None, [_c_void_p] * 3 + [_c_int32] * 4 + [_c_float, _c_int32, _c_void_p]),
     "mgpuFusedMHABF16CuSeqlens": (None, [_c_void_p] * 3 + [_c_int32] * 4 + [_c_float, _c_int32, _c_void_p]),
-    "mgpuFusedMHAF16Profile": (_c_int64, [_c_void_p, _c_void_p] + [_c_int32] * 3 + [_c_float, _c_void_p, _c_void_p]),
     "mgpuCastF32ToF16": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
     "mgpuCastF16ToF32": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
     "mgpuCastF32ToBF16": (None, [_c_void_p, _c_void_p, _c_size_t, _c_void_p]),
@@ -71,7 +70,6 @@ OPS_SIGNATURES = {
     "mgpuPool2d": (None, [_c_void_p] * 2 + [_c_int64] * 15 + [_c_void_p]),
     "mgpuMatmulExF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuMatmulExBF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
-    "mgpuMatmulExTune": (_c_int32, [_c_int32] + [_c_int64] * 3 + [_c_int32] * 3),
     "mgpuGemmMfmaF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuGemmMfmaBF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuMatmulExF32": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
@@ -135,6 +133,33 @@ def runtime() -> ctypes.CDLL:
     if _runtime is None:
         _runtime = _load(RUNTIME_LIB, RUNTIME_SIGNATURES)
     return _runtime
+
+
+BENCH_LIB = os.path.join(LIB_DIR, "libmgpu_bench_loops.so")
+_bench = None
+
+
+def bench_loops() -> ctypes.CDLL:
+    """The benchmark's launch loops, ceiling probes, attention profile entry and GEMM tuner
+    (measurement plumbing, not part of the kernel library)."""
+    global _bench
+    if _bench is None:
+        if not os.path.exists(BENCH_LIB):
+            raise MgpuError(f"{BENCH_LIB} is not built")
+        ops(init=False)  # the loops call into the kernel library
+        lib = ctypes.CDLL(BENCH_LIB)
+        f32 = ctypes.c_float
+        for name in ("mgpuBenchLayerNormF32", "mgpuBenchLayerNormF16", "mgpuBenchAddF32", "mgpuBenchFusedMHAF16",
+                     "mgpuBenchBertEncoderLayerF16", "mgpuProbeCopy", "mgpuProbeCombine", "mgpuProbeMfma",
+                     "mgpuProbeFmhaLoop", "mgpuProbeLdsRead"):
+            getattr(lib, name).restype = f32
+        lib.mgpuBenchFusedMHAF16Profile.restype = _c_int64
+        lib.mgpuBenchFusedMHAF16Profile.argtypes = [_c_void_p, _c_void_p] + [_c_int32] * 3 + [_c_float, _c_void_p,
+                                                                                               _c_void_p]
+        lib.mgpuBenchTuneMatmulEx.restype = _c_int32
+        lib.mgpuBenchTuneMatmulEx.argtypes = [_c_int32] + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p, _c_void_p]
+        _bench = lib
+    return _bench
 
 
 def ops(init: bool = True) -> ctypes.CDLL:
@@ -381,14 +406,14 @@ def pool2d(x, kernel, pad=(0, 0, 0, 0), stride=(1, 1), method="max", stream=None
 
 
 def decoding_context_layer(x, wqkv, wo, bo, w1, b1, w2, b2, heads: int, causal: bool = True,
-                           relu: bool = True, stream=None):
+                           relu: bool = True, norm_first: bool = True, stream=None):
     import torch
     B, S, d = x.shape
     ffn = w1.shape[1]
     out = torch.empty_like(x)
     lib = ops()
     lib.mgpuLLMDecodingContextLayer(_ptr(x), _ptr(wqkv), _ptr(wo), _ptr(bo), _ptr(w1), _ptr(b1),
-                                    _ptr(w2), _ptr(b2), _ptr(out), B, S, d, ffn, heads, True,
+                                    _ptr(w2), _ptr(b2), _ptr(out), B, S, d, ffn, heads, norm_first,
                                     causal, relu, _stream_handle(stream))
     _check(lib)
     return out

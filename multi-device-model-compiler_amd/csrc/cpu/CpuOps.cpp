@@ -400,7 +400,7 @@ void mcpuMatmulExF16(void *input, void *weight, void *bias, void *output, void *
 void mcpuLLMDecodingContextLayer(float *input, float *qkv, float *gemm_weight, float *gemm_bias, float *ffn1_weight,
                                  float *ffn1_bias, float *ffn2_weight, float *ffn2_bias, float *output, int64_t batch,
                                  int64_t seq_len, int64_t d_model, int64_t feed_forward_dim, int64_t head_num,
-                                 bool /*norm_first*/, bool is_casual, bool is_relu) {
+                                 bool norm_first, bool is_casual, bool is_relu) {
   const int64_t M = batch * seq_len, d = d_model, ffn = feed_forward_dim;
   if (M <= 0 || d <= 0 || ffn <= 0 || head_num <= 0 || d % head_num) return;
   auto half = [](const float *src, size_t n) {
@@ -414,16 +414,30 @@ void mcpuLLMDecodingContextLayer(float *input, float *qkv, float *gemm_weight, f
                               w2 = half(ffn2_weight, (size_t)ffn * d), b2 = half(ffn2_bias, (size_t)d);
   std::vector<uint16_t> ln((size_t)M * d), packed((size_t)M * 3 * d), ctx((size_t)M * d), proj((size_t)M * d),
       y((size_t)M * d), f((size_t)M * ffn), o((size_t)M * d);
-  mcpuLayerNormF16(x.data(), nullptr, nullptr, ln.data(), 1e-5f, (int32_t)M, (int32_t)d);
-  matmulExF16(ln.data(), wqkv.data(), nullptr, packed.data(), nullptr, M, 3 * d, d, 0);
   const int64_t dh = d / head_num;
-  mcpuFusedMHAF16(packed.data(), nullptr, ctx.data(), (int32_t)batch, (int32_t)seq_len, (int32_t)head_num, (int32_t)dh,
-                  1.0f / std::sqrt((float)dh), is_casual ? 1 : 0);
-  matmulExF16(ctx.data(), wo.data(), bo.data(), proj.data(), nullptr, M, d, d, 0);
-  mcpuAddResidualPreLayerNormF16(proj.data(), x.data(), nullptr, nullptr, y.data(), ln.data(), 1e-5f, (int32_t)M,
-                                 (int32_t)d);
-  matmulExF16(ln.data(), w1.data(), b1.data(), f.data(), nullptr, M, ffn, d, is_relu ? 1 : 2);
-  matmulExF16(f.data(), w2.data(), b2.data(), o.data(), y.data(), M, d, ffn, 0);
+  const int act = is_relu ? 1 : 2;
+  if (norm_first) { // y = x + proj(attention(LN(x))), out = y + ffn(LN(y))
+    mcpuLayerNormF16(x.data(), nullptr, nullptr, ln.data(), 1e-5f, (int32_t)M, (int32_t)d);
+    matmulExF16(ln.data(), wqkv.data(), nullptr, packed.data(), nullptr, M, 3 * d, d, 0);
+    mcpuFusedMHAF16(packed.data(), nullptr, ctx.data(), (int32_t)batch, (int32_t)seq_len, (int32_t)head_num,
+                    (int32_t)dh, 1.0f / std::sqrt((float)dh), is_casual ? 1 : 0);
+    matmulExF16(ctx.data(), wo.data(), bo.data(), proj.data(), nullptr, M, d, d, 0);
+    mcpuAddResidualPreLayerNormF16(proj.data(), x.data(), nullptr, nullptr, y.data(), ln.data(), 1e-5f, (int32_t)M,
+                                   (int32_t)d);
+    matmulExF16(ln.data(), w1.data(), b1.data(), f.data(), nullptr, M, ffn, d, act);
+    matmulExF16(f.data(), w2.data(), b2.data(), o.data(), y.data(), M, d, ffn, 0);
+  } else { // post-LN: h = LN(x + proj(attention(x))), out = LN(h + ffn(h))
+    matmulExF16(x.data(), wqkv.data(), nullptr, packed.data(), nullptr, M, 3 * d, d, 0);
+    mcpuFusedMHAF16(packed.data(), nullptr, ctx.data(), (int32_t)batch, (int32_t)seq_len, (int32_t)head_num,
+                    (int32_t)dh, 1.0f / std::sqrt((float)dh), is_casual ? 1 : 0);
+    matmulExF16(ctx.data(), wo.data(), bo.data(), proj.data(), nullptr, M, d, d, 0);
+    mcpuAddResidualPreLayerNormF16(proj.data(), x.data(), nullptr, nullptr, ln.data(), y.data(), 1e-5f, (int32_t)M,
+                                   (int32_t)d); // y = h; ln takes the rounded sum nobody reads
+    matmulExF16(y.data(), w1.data(), b1.data(), f.data(), nullptr, M, ffn, d, act);
+    matmulExF16(f.data(), w2.data(), b2.data(), proj.data(), nullptr, M, d, ffn, 0);
+    mcpuAddResidualPreLayerNormF16(proj.data(), y.data(), nullptr, nullptr, ln.data(), o.data(), 1e-5f, (int32_t)M,
+                                   (int32_t)d);
+  }
   mcpuCastF16ToF32(output, o.data(), (size_t)M * d);
 }
 

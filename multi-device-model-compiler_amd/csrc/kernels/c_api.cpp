@@ -33,7 +33,6 @@ template <typename F> void guarded(F &&f) noexcept {
 }
 
 inline hipStream_t S(mgpuStream_t s) { return reinterpret_cast<hipStream_t>(s); }
-inline hipStream_t S_(mgpuStream_t s) { return reinterpret_cast<hipStream_t>(s); } // where a parameter is called S
 
 } // namespace
 
@@ -234,13 +233,6 @@ void mgpuFusedMHABF16CuSeqlens(const void *qkv, const int32_t *cu_seqlens, void 
   });
 }
 
-int64_t mgpuFusedMHAF16Profile(const void *qkv, void *out, int32_t B, int32_t S, int32_t H, float scale,
-                               uint64_t *stamps, mgpuStream_t stream) {
-  int64_t blocks = 0;
-  guarded([&] { blocks = mgpu::fusedMHAProfile(qkv, out, B, S, H, scale, stamps, S_(stream)); });
-  return blocks;
-}
-
 void mgpuCastF32ToF16(void *dst, const float *src, size_t size, mgpuStream_t stream) {
   guarded([&] { mgpu::castF32ToF16(dst, src, size, S(stream)); });
 }
@@ -327,15 +319,6 @@ void mgpuGemmMfmaBF16(void *input, void *weight, void *bias, void *output, void 
     gemmMfmaChecked(mgpu::DType::BF16, input, weight, bias, output, residual, M, N, K, hasBias, hasRelu, hasResidual,
                     S(stream));
   });
-}
-int32_t mgpuMatmulExTune(int32_t dtype, int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
-                         int32_t hasResidual) {
-  int32_t kept = -1;
-  guarded([&] {
-    if (dtype < 0 || dtype > 2) mgpu::fail("mgpuMatmulExTune: dtype is 0 (fp32), 1 (fp16) or 2 (bf16)");
-    kept = mgpu::tuneMatmulEx(static_cast<mgpu::DType>(dtype), M, N, K, hasBias != 0, hasRelu, hasResidual != 0) ? 1 : 0;
-  });
-  return kept;
 }
 void mgpuMatmulExBF16(void *input, void *weight, void *bias, void *output, void *residual,
                       int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,

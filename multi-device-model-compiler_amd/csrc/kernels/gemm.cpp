@@ -15,12 +15,9 @@
 //    table decided offline (gemm_table.inc, written by `bench.py --tune-gemm`
 //    from measurements on an MI355X) and, for shapes the table does not hold,
 //    from a fixed rule; the library runs the heuristic's first algorithm.
-//    MGPU_GEMM_KERNEL=library or =mfma in the environment overrides both.  A
-//    caller who wants a shape measured on its own device asks for it
-//    explicitly with tuneMatmulEx (mgpuMatmulExTune in the C ABI), outside any
-//    stream capture: that call allocates scratch operands, times the
-//    library's candidates and the hand-written kernel, and keeps the winner
-//    for the rest of the process;
+//    MGPU_GEMM_KERNEL=library or =mfma in the environment overrides both.
+//    Nothing in this library measures anything: the tuner that writes the
+//    table lives with the benchmark's launch loops;
 //  * the library's workspace is per caller stream (allocated on a stream's
 //    first library GEMM outside a capture), so GEMMs on different streams never
 //    share one; a stream first seen under capture gets an algorithm that needs
@@ -52,13 +49,19 @@ bool isCapturing(hipStream_t s) {
   return hipStreamIsCapturing(s, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone;
 }
 
-// The stream's workspace; null when it has none yet and none can be made now (capture).
+// The stream's workspace; null when it has none yet and none can be made now (the stream
+// is capturing, or the allocation failed).  Workspaces are kept per stream handle until
+// gemmDeinit(); a caller that creates and destroys streams without end should run its
+// GEMMs on a bounded set of them.
 void *workspaceFor(hipStream_t s) {
   auto it = workspaceOf.find(s);
   if (it != workspaceOf.end()) return it->second;
   if (isCapturing(s)) return nullptr;
   void *ws = nullptr;
-  MGPU_CHECK_HIP(hipMalloc(&ws, workspaceSize));
+  if (hipMalloc(&ws, workspaceSize) != hipSuccess) { // out of memory, or another stream is capturing
+    (void)hipGetLastError();
+    return nullptr; // the caller falls back to an algorithm that needs no workspace; asked again next time
+  }
   workspaceOf[s] = ws;
   return ws;
 }
@@ -131,133 +134,16 @@ void destroyPlan(Plan &p) {
   p = Plan{};
 }
 
-constexpr int kCandidates = 64; // heuristic answers asked for and screened
-constexpr int kFinalists = 4;   // re-timed at length after the screening pass
-
-// Times the candidates on scratch operands of the plan's shape (its own stream,
-// its own buffers: the caller's data and stream are not touched) and returns
-// the index of the fastest; 0 when nothing could be measured.  *handWritten
-// says whether the hand-written kernel beat it (with the separate GELU pass
-// counted on the library's side).
-int fastestCandidate(const Plan &p, const hipblasLtMatmulHeuristicResult_t *results, int count, DType dt,
-                     int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual,
-                     bool *handWritten) {
-  const size_t eb = dt == DType::F32 ? 4 : 2;
-  void *in = nullptr, *w = nullptr, *out = nullptr, *bias = nullptr, *workspace = nullptr;
-  hipStream_t s = nullptr;
-  hipEvent_t e0 = nullptr, e1 = nullptr;
-  int best = 0;
-  const bool ready = hipMalloc(&in, (size_t)M * K * eb) == hipSuccess && hipMalloc(&w, (size_t)K * N * eb) == hipSuccess &&
-                     hipMalloc(&out, (size_t)M * N * eb) == hipSuccess && hipMalloc(&bias, (size_t)N * eb) == hipSuccess &&
-                     hipMalloc(&workspace, workspaceSize) == hipSuccess &&
-                     hipStreamCreate(&s) == hipSuccess && hipEventCreate(&e0) == hipSuccess &&
-                     hipEventCreate(&e1) == hipSuccess;
-  if (ready) {
-    // 0x3c bytes: 1.06 as fp16, 0.0115 as fp32, finite in every type
-    (void)hipMemsetAsync(in, 0x3c, (size_t)M * K * eb, s);
-    (void)hipMemsetAsync(w, 0x3c, (size_t)K * N * eb, s);
-    (void)hipMemsetAsync(out, 0x3c, (size_t)M * N * eb, s);
-    (void)hipMemsetAsync(bias, 0x3c, (size_t)N * eb, s);
-    if (hasBias)
-      (void)hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
-    const float alpha = 1.0f, beta = hasResidual ? 1.0f : 0.0f;
-    // reps launches of candidate c between two events, after one untimed launch; < 0 on failure
-    auto timeCandidate = [&](int c, int reps) -> float {
-      bool ok = true;
-      for (int rep = 0; rep <= reps && ok; rep++) {
-        if (rep == 1) (void)hipEventRecord(e0, s);
-        ok = hipblasLtMatmul(ltHandle, p.op, &alpha, w, p.a, in, p.b, &beta, out, p.d, out, p.d, &results[c].algo,
-                             workspace, workspaceSize, s) == HIPBLAS_STATUS_SUCCESS;
-      }
-      float ms = 0.0f;
-      if (!ok || hipEventRecord(e1, s) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
-          hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
-        return -1.0f;
-      return ms / reps;
-    };
-    // Screening: three launches each; the kFinalists fastest go on.
-    std::vector<std::pair<float, int>> screened;
-    for (int c = 0; c < count; c++) {
-      if (results[c].state != HIPBLAS_STATUS_SUCCESS || results[c].workspaceSize > workspaceSize) continue;
-      const float ms = timeCandidate(c, 3);
-      if (ms >= 0.0f) screened.emplace_back(ms, c);
-    }
-    std::sort(screened.begin(), screened.end());
-    // Final: twenty launches each.
-    float bestMs = -1.0f;
-    for (size_t i = 0; i < screened.size() && i < (size_t)kFinalists; i++) {
-      const float ms = timeCandidate(screened[i].second, 20);
-      if (ms >= 0.0f && (bestMs < 0.0f || ms < bestMs)) {
-        bestMs = ms;
-        best = screened[i].second;
-      }
-    }
-    // The hand-written kernel on the same operands (`out` doubles as the residual).
-    const void *biasArg = hasBias ? bias : nullptr, *resArg = hasResidual ? out : nullptr;
-    if (bestMs >= 0.0f && gemmMfmaSupports(dt, in, w, biasArg, resArg, out, M, N, K)) {
-      // Both paths in alternating runs of twenty launches, three runs each, so that
-      // they meet the same clocks: a lone burst of a kernel that has the device to
-      // itself for a millisecond runs faster than the same kernel in a layer.
-      auto timeLoop = [&](auto &&launchOnce) -> float {
-        try {
-          launchOnce();
-          (void)hipEventRecord(e0, s);
-          for (int rep = 0; rep < 20; rep++) launchOnce();
-        } catch (const std::exception &) {
-          return -1.0f;
-        }
-        float ms = 0.0f;
-        if (hipEventRecord(e1, s) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
-            hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
-          return -1.0f;
-        return ms;
-      };
-      const float alpha1 = 1.0f, beta1 = hasResidual ? 1.0f : 0.0f;
-      auto libraryOnce = [&] {
-        if (hipblasLtMatmul(ltHandle, p.op, &alpha1, w, p.a, in, p.b, &beta1, out, p.d, out, p.d, &results[best].algo,
-                            workspace, workspaceSize, s) != HIPBLAS_STATUS_SUCCESS)
-          throw std::runtime_error("hipblasLtMatmul");
-        if (act == ACT_GELU) {
-          if (dt == DType::F16) geluInPlaceF16(out, (size_t)M * N, s);
-          else geluInPlaceBF16(out, (size_t)M * N, s);
-        }
-      };
-      auto mfmaOnce = [&] { gemmMfma(dt, in, w, biasArg, resArg, out, M, N, K, act, s); };
-      float libraryMs = 0.0f, mfmaMs = 0.0f;
-      bool ok = true;
-      for (int round = 0; round < 3 && ok; round++) {
-        const float l = timeLoop(libraryOnce), m = timeLoop(mfmaOnce);
-        ok = l >= 0.0f && m >= 0.0f;
-        libraryMs += l;
-        mfmaMs += m;
-      }
-      // three per cent of margin: a tie goes to the library
-      *handWritten = ok && mfmaMs < 0.97f * libraryMs;
-    }
-    (void)hipStreamSynchronize(s);
-  }
-  if (e0) (void)hipEventDestroy(e0);
-  if (e1) (void)hipEventDestroy(e1);
-  if (s) (void)hipStreamDestroy(s);
-  for (void *ptr : {in, w, out, bias, workspace})
-    if (ptr) (void)hipFree(ptr);
-  (void)hipGetLastError();
-  return best;
-}
+constexpr int kCandidates = 16; // heuristic answers looked through for one that needs no workspace
 
 // Builds (once per shape, flags and type) the library's descriptors and picks its
 // algorithms; decides which kernel serves the shape.  No measurement, no allocation
-// beyond the library's host-side descriptors.  With `tune` the caller has asked for the
-// measurement (tuneMatmulEx).
-Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual, bool tune) {
+// beyond the library's host-side descriptors.
+Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual) {
   const bool relu = act == ACT_RELU;
   const Key key{M, N, K, (int)hasBias, act, (int)hasResidual, (int)dt};
   auto it = plans.find(key);
-  if (it != plans.end() && !tune) return it->second;
-  if (it != plans.end()) {
-    destroyPlan(it->second);
-    plans.erase(it);
-  }
+  if (it != plans.end()) return it->second;
 
   Plan p;
   const hipDataType t = dataType(dt);
@@ -312,11 +198,6 @@ Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, 
     if (e.dt == (int)dt && e.M == M && e.N == N && e.K == K && e.hasBias == (int)hasBias && e.act == act &&
         e.hasResidual == (int)hasResidual)
       p.handWritten = mfmaShape && e.handWritten != 0;
-  if (tune) {
-    const int best = fastestCandidate(p, results, returned, dt, M, N, K, hasBias, act, hasResidual, &p.handWritten);
-    p.algo = results[best].algo;
-    p.algoWorkspace = results[best].workspaceSize;
-  }
   if (forcedKernel()) p.handWritten = forcedKernel() == 2;
   return plans.emplace(key, p).first->second;
 }
@@ -354,7 +235,7 @@ void matmulEx(DType dt, const void *input, const void *weight, const void *bias,
     fail("matmul: an activation cannot be combined with a residual");
 
   std::lock_guard<std::mutex> lock(planMutex);
-  const Plan &p = getPlan(dt, M, N, K, hasBias, act, hasResidual, false);
+  const Plan &p = getPlan(dt, M, N, K, hasBias, act, hasResidual);
   if (p.handWritten && gemmMfmaSupports(dt, input, weight, hasBias ? bias : nullptr,
                                         hasResidual ? residual : nullptr, output, M, N, K)) {
     gemmMfma(dt, input, weight, hasBias ? bias : nullptr, hasResidual ? residual : nullptr, output, M, N, K, act,
@@ -370,7 +251,7 @@ void matmulEx(DType dt, const void *input, const void *weight, const void *bias,
   void *workspace = p.algoWorkspace ? workspaceFor(stream) : nullptr;
   const hipblasLtMatmulAlgo_t *algo = &p.algo;
   if (p.algoWorkspace && !workspace) {
-    if (!p.hasNoWs) fail("matmul: the library needs a workspace for this shape; run it once on this stream before capturing");
+    if (!p.hasNoWs) fail("matmul: the library needs a workspace for this shape and none could be allocated now (stream capture or out of memory); run it once on this stream before capturing");
     algo = &p.algoNoWs;
   }
   MGPU_CHECK_BLAS(hipblasLtMatmul(ltHandle, p.op, &alpha, weight, p.a, input, p.b, &beta,
@@ -384,19 +265,6 @@ void matmulEx(DType dt, const void *input, const void *weight, const void *bias,
     else
       geluInPlaceF32(static_cast<float *>(output), (size_t)M * N, stream);
   }
-}
-
-// Measures, on this device and on scratch operands of the shape, the library's top
-// candidates and the hand-written kernel, and keeps the faster path for the rest of the
-// process.  Synchronous, allocates and frees device memory: never call it under stream
-// capture or from a path that must only enqueue.  Returns true when the hand-written
-// kernel was kept.
-bool tuneMatmulEx(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual) {
-  if (M <= 0 || N <= 0 || K <= 0) fail("tuneMatmulEx: bad shape");
-  if (!ltHandle) fail("tuneMatmulEx: gpuOpsInit() has not been called");
-  if (act < ACT_NONE || act > ACT_GELU || (act != ACT_NONE && hasResidual)) fail("tuneMatmulEx: bad epilogue");
-  std::lock_guard<std::mutex> lock(planMutex);
-  return getPlan(dt, M, N, K, hasBias, act, hasResidual, true).handWritten;
 }
 
 } // namespace mgpu

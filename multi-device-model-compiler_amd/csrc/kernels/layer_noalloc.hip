@@ -38,7 +38,9 @@ constexpr int kMaxDevices = 64;
 void *scratchAddress[kMaxDevices] = {};
 std::mutex scratchAddressMutex;
 
-// Address of `scratch` on the current device, looked up on first use there.
+// Address of `scratch` on the current device, looked up on first use there.  The caller's
+// stream must belong to the current device (as for every entry point of this library: the
+// kernels are launched on the stream, the scratch address is the current device's).
 unsigned char *scratchOnCurrentDevice() {
   int dev = -1;
   MGPU_CHECK_HIP(hipGetDevice(&dev));
@@ -96,20 +98,33 @@ void bertEncoderLayerF16NoAlloc(const void *x, const void *wqkv, const void *bqk
   void *qkv = base, *ctx = base + qkvBytes, *f = base;
   void *proj = base + headBytes, *h1 = base + headBytes + rowBytes;
 
-  auto gemm = [&](const void *in, const void *w, const void *bias, void *o, int64_t N, int64_t K, int act) {
-    if (!gemmMfmaSupports(DType::F16, in, w, bias, nullptr, o, M, N, K))
+  // Everything that can reject the call is checked before the first launch, so that a rejected
+  // call enqueues nothing (under capture: leaves no partial graph).
+  struct Gemm {
+    const void *in, *w, *bias;
+    void *o;
+    int64_t N, K;
+    int act;
+  };
+  const Gemm gemms[4] = {{x, wqkv, bqkv, qkv, 3 * d, d, ACT_NONE},
+                         {ctx, wo, bo, proj, d, d, ACT_NONE},
+                         {h1, w1, b1, f, ffn, d, ACT_GELU},
+                         {f, w2, b2, proj, d, ffn, ACT_NONE}};
+  for (const Gemm &g : gemms)
+    if (!gemmMfmaSupports(DType::F16, g.in, g.w, g.bias, nullptr, g.o, M, g.N, g.K))
       fail(std::string(name) + ": batch * seq_len must be a multiple of 128, every GEMM width a multiple of 128 or 96, "
                                "every depth a multiple of 32, and the operands 16-byte aligned");
-    gemmMfma(DType::F16, in, w, bias, nullptr, o, M, N, K, act, stream);
-  };
+  if (!aligned16(x) || !aligned16(out) || !aligned16(gamma1) || !aligned16(beta1) || !aligned16(gamma2) || !aligned16(beta2))
+    fail(std::string(name) + ": x, out and the LayerNorm vectors must be 16-byte aligned");
+  auto gemm = [&](const Gemm &g) { gemmMfma(DType::F16, g.in, g.w, g.bias, nullptr, g.o, M, g.N, g.K, g.act, stream); };
 
-  gemm(x, wqkv, bqkv, qkv, 3 * d, d, ACT_NONE);
+  gemm(gemms[0]);
   fusedMHA(DType::F16, qkv, seqlens, ctx, (int)B, (int)S, (int)H, (int)(d / H), 1.0f / sqrtf((float)(d / H)), false,
            stream);
-  gemm(ctx, wo, bo, proj, d, d, ACT_NONE);
+  gemm(gemms[1]);
   layerNorm(DType::F16, proj, x, gamma1, beta1, nullptr, h1, eps, (int)M, (int)d, stream);
-  gemm(h1, w1, b1, f, ffn, d, ACT_GELU);
-  gemm(f, w2, b2, proj, d, ffn, ACT_NONE);
+  gemm(gemms[2]);
+  gemm(gemms[3]);
   layerNorm(DType::F16, proj, h1, gamma2, beta2, nullptr, out, eps, (int)M, (int)d, stream);
 }
 

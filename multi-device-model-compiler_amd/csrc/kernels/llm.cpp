@@ -6,8 +6,10 @@
 // Kept from the reference: the dataflow (pre-LN, gamma = 1 / beta = 0
 // LayerNorms at eps 1e-5, packed-QKV attention, bias epilogues, residual
 // through the GEMM's C operand).  Changed on purpose:
-//  * head_num, is_casual and is_relu are honoured (the reference ignores them
-//    and runs 8 heads x 128, causal, ReLU: LLM.cu:18-19,79-81,119-121);
+//  * head_num, norm_first, is_casual and is_relu are honoured (the reference
+//    ignores them and runs 8 heads x 128, pre-LN, causal, ReLU:
+//    LLM.cu:18-19,79-81,119-121); norm_first = false is the post-LN ordering
+//    of the same blocks;
 //  * one arena instead of 12 allocations and frees per call, and the arena is
 //    kept per caller stream between calls (an allocation and a free per call
 //    cost 14 us of host time, about a tenth of a BERT-base layer): it grows to
@@ -169,7 +171,7 @@ void llmDeinit() {
 void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *gemm_bias,
                           float *ffn1_weight, float *ffn1_bias, float *ffn2_weight,
                           float *ffn2_bias, float *output, int64_t batch, int64_t seq_len,
-                          int64_t d_model, int64_t ffn, int64_t heads, bool /*norm_first*/,
+                          int64_t d_model, int64_t ffn, int64_t heads, bool norm_first,
                           bool causal, bool relu, hipStream_t stream) {
   if (!initialised) fail("mgpuLLMDecodingContextLayer: gpuOpsInit() has not been called");
   if (batch < 0 || seq_len < 0 || d_model <= 0 || ffn <= 0 || heads <= 0)
@@ -238,35 +240,63 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
     fillF16(arena.at(oBeta), d, 0.0f, stream);
   }
 
-  // fp16 copy of the input (the residual of the second LayerNorm) and its
-  // LayerNorm: one kernel where the width allows, else the reference's two.
-  if (!castLayerNormF32ToF16(input, gamma, beta, arena.at(oX), arena.at(oLn), 1e-5f, (int)M, (int)d, stream)) {
+  if (norm_first) {
+    // y = x + proj(attention(LN(x))), out = y + ffn(LN(y))
+    // fp16 copy of the input (the residual of the second LayerNorm) and its
+    // LayerNorm: one kernel where the width allows, else the reference's two.
+    if (!castLayerNormF32ToF16(input, gamma, beta, arena.at(oX), arena.at(oLn), 1e-5f, (int)M, (int)d, stream)) {
+      castF32ToF16(arena.at(oX), input, M * d, stream);
+      layerNorm(DType::F16, arena.at(oX), nullptr, gamma, beta, nullptr, arena.at(oLn), 1e-5f, (int)M, (int)d, stream);
+    }
+
+    join(0);
+    matmulEx(DType::F16, arena.at(oLn), arena.at(oWqkv), nullptr, arena.at(oQkv), nullptr, M, 3 * d,
+             d, false, ACT_NONE, false, stream);
+
+    // Attention context overwrites the first LayerNorm output, like the reference.
+    fusedMHA(DType::F16, arena.at(oQkv), nullptr, arena.at(oLn), (int)batch, (int)seq_len,
+             (int)heads, (int)(d_model / heads), 1.0f / sqrtf((float)(d_model / heads)), causal, stream);
+
+    join(1);
+    matmulEx(DType::F16, arena.at(oLn), arena.at(oWo), arena.at(oBo), arena.at(oProj), nullptr, M, d,
+             d, true, ACT_NONE, false, stream);
+
+    layerNorm(DType::F16, arena.at(oProj), arena.at(oX), gamma, beta, arena.at(oY), arena.at(oLn), 1e-5f, (int)M,
+              (int)d, stream);
+
+    join(2);
+    matmulEx(DType::F16, arena.at(oLn), arena.at(oW1), arena.at(oB1), arena.at(oF), nullptr, M, ffn,
+             d, true, relu ? ACT_RELU : ACT_GELU, false, stream);
+
+    join(3); // also the join of the fork: nothing of this call is left on the side stream after it
+    matmulEx(DType::F16, arena.at(oF), arena.at(oW2), arena.at(oB2), arena.at(oOut), arena.at(oY), M,
+             d, ffn, true, ACT_NONE, true, stream);
+  } else {
+    // norm_first = false, the post-LN ordering of the same blocks (the reference declares the
+    // flag, Ops.h:43-48, and never reads it):  h = LN(x + proj(attention(x))),
+    // out = LN(h + ffn(h)), both LayerNorms with gamma = 1 / beta = 0 at eps 1e-5 like the
+    // pre-LN ones, every intermediate stored in fp16 where the pre-LN path stores it.
     castF32ToF16(arena.at(oX), input, M * d, stream);
-    layerNorm(DType::F16, arena.at(oX), nullptr, gamma, beta, nullptr, arena.at(oLn), 1e-5f, (int)M, (int)d, stream);
+    join(0);
+    matmulEx(DType::F16, arena.at(oX), arena.at(oWqkv), nullptr, arena.at(oQkv), nullptr, M, 3 * d,
+             d, false, ACT_NONE, false, stream);
+    fusedMHA(DType::F16, arena.at(oQkv), nullptr, arena.at(oLn), (int)batch, (int)seq_len,
+             (int)heads, (int)(d_model / heads), 1.0f / sqrtf((float)(d_model / heads)), causal, stream);
+    join(1);
+    matmulEx(DType::F16, arena.at(oLn), arena.at(oWo), arena.at(oBo), arena.at(oProj), nullptr, M, d,
+             d, true, ACT_NONE, false, stream);
+    // h (in oY) = LN(proj + x); the rounded sum is not needed again
+    layerNorm(DType::F16, arena.at(oProj), arena.at(oX), gamma, beta, nullptr, arena.at(oY), 1e-5f, (int)M,
+              (int)d, stream);
+    join(2);
+    matmulEx(DType::F16, arena.at(oY), arena.at(oW1), arena.at(oB1), arena.at(oF), nullptr, M, ffn,
+             d, true, relu ? ACT_RELU : ACT_GELU, false, stream);
+    join(3);
+    matmulEx(DType::F16, arena.at(oF), arena.at(oW2), arena.at(oB2), arena.at(oProj), nullptr, M,
+             d, ffn, true, ACT_NONE, false, stream);
+    layerNorm(DType::F16, arena.at(oProj), arena.at(oY), gamma, beta, nullptr, arena.at(oOut), 1e-5f, (int)M,
+              (int)d, stream);
   }
-
-  join(0);
-  matmulEx(DType::F16, arena.at(oLn), arena.at(oWqkv), nullptr, arena.at(oQkv), nullptr, M, 3 * d,
-           d, false, ACT_NONE, false, stream);
-
-  // Attention context overwrites the first LayerNorm output, like the reference.
-  fusedMHA(DType::F16, arena.at(oQkv), nullptr, arena.at(oLn), (int)batch, (int)seq_len,
-           (int)heads, (int)(d_model / heads), 1.0f / sqrtf((float)(d_model / heads)), causal, stream);
-
-  join(1);
-  matmulEx(DType::F16, arena.at(oLn), arena.at(oWo), arena.at(oBo), arena.at(oProj), nullptr, M, d,
-           d, true, ACT_NONE, false, stream);
-
-  layerNorm(DType::F16, arena.at(oProj), arena.at(oX), gamma, beta, arena.at(oY), arena.at(oLn), 1e-5f, (int)M,
-            (int)d, stream);
-
-  join(2);
-  matmulEx(DType::F16, arena.at(oLn), arena.at(oW1), arena.at(oB1), arena.at(oF), nullptr, M, ffn,
-           d, true, relu ? ACT_RELU : ACT_GELU, false, stream);
-
-  join(3); // also the join of the fork: nothing of this call is left on the side stream after it
-  matmulEx(DType::F16, arena.at(oF), arena.at(oW2), arena.at(oB2), arena.at(oOut), arena.at(oY), M,
-           d, ffn, true, ACT_NONE, true, stream);
 
   castF16ToF32(output, arena.at(oOut), M * d, stream);
   arena.release(stream);

@@ -34,13 +34,6 @@ void fusedMHA(DType dt, const void *qkv, const int32_t *seqlens, void *out, int 
 void fusedMHACuSeqlens(DType dt, const void *qkv, const int32_t *cuSeqlens, void *out, int B, int maxS, int H,
                        int D, float scale, bool causal, hipStream_t stream);
 
-// The fp16 head_dim-64 unmasked kernel with per-block clock stamps: ten uint64 per
-// block (shader clock at entry, first tile landed, last tile done, stores issued;
-// constant-rate clock at entry and exit; clocks spent waiting for tiles, in the
-// score MFMAs, in the softmax, in the P.V MFMAs).  Returns the number of blocks.
-int64_t fusedMHAProfile(const void *qkv, void *out, int B, int S, int H, float scale, uint64_t *stamps,
-                        hipStream_t stream);
-
 void castF32ToF16(void *dst, const float *src, size_t size, hipStream_t stream);
 void castF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream);
 void castF32ToBF16(void *dst, const float *src, size_t size, hipStream_t stream);
@@ -59,11 +52,6 @@ void gemmDeinit();
 void matmulEx(DType dt, const void *input, const void *weight, const void *bias, void *output,
               const void *residual, int64_t M, int64_t N, int64_t K, bool hasBias, int act,
               bool hasResidual, hipStream_t stream);
-
-// Explicit, synchronous measurement of a shape (library candidates against the
-// hand-written kernel); the result replaces the table's / the rule's choice for
-// the rest of the process.  Not for capture or enqueue-only paths.
-bool tuneMatmulEx(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual);
 
 // Hand-written MFMA GEMM (gemm_mfma.hip): fp16 / bf16, M a multiple of 128, N of
 // 128 or 96, K of 32, 16-byte aligned operands; bias and residual may be null.

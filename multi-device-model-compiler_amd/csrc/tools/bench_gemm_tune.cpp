@@ -1,0 +1,182 @@
+// The GEMM tuner behind `bench.py --tune-gemm`: for one shape and epilogue it times
+// hipBLASLt's candidate algorithms (the [K, N] row-major weight of mgpuMatmulEx, fp32
+// accumulation, bias / ReLU epilogue, a separate exact-erf GELU pass where there is one)
+// against the hand-written MFMA kernel, on scratch operands, its own stream and its own
+// workspace, and says which side won.  Its answers are the rows of
+// csrc/kernels/gemm_table.inc; the kernel library itself never measures.
+// Measurement plumbing only: nothing here is part of the kernel library.
+#include "mgpu_ops_internal.hpp"
+
+#include <hip/hip_runtime.h>
+#include <hipblaslt/hipblaslt.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <stdexcept>
+#include <utility>
+#include <vector>
+
+namespace {
+
+constexpr size_t kWorkspace = 32u * 1024u * 1024u;
+constexpr int kCandidates = 64; // heuristic answers asked for and screened
+constexpr int kFinalists = 4;   // re-timed at length after the screening pass
+
+struct Scratch {
+  void *in = nullptr, *w = nullptr, *out = nullptr, *bias = nullptr, *workspace = nullptr;
+  hipStream_t s = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipblasLtHandle_t lt = nullptr;
+  hipblasLtMatmulDesc_t op = nullptr;
+  hipblasLtMatrixLayout_t a = nullptr, b = nullptr, d = nullptr;
+  ~Scratch() {
+    if (d) hipblasLtMatrixLayoutDestroy(d);
+    if (b) hipblasLtMatrixLayoutDestroy(b);
+    if (a) hipblasLtMatrixLayoutDestroy(a);
+    if (op) hipblasLtMatmulDescDestroy(op);
+    if (lt) hipblasLtDestroy(lt);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (s) (void)hipStreamDestroy(s);
+    for (void *p : {in, w, out, bias, workspace})
+      if (p) (void)hipFree(p);
+    (void)hipGetLastError();
+  }
+};
+
+} // namespace
+
+extern "C" {
+
+// dtype: 0 fp32, 1 fp16, 2 bf16; act: 0 none, 1 ReLU, 2 GELU.  Returns 1 when the hand-written
+// kernel is faster by more than three per cent, 0 when the library is kept (also for shapes the
+// hand-written kernel does not take), -1 when nothing could be measured.  *libraryUs / *mfmaUs
+// receive the microseconds per launch of the library's best candidate (plus the GELU pass) and
+// of the hand-written kernel (0 where it does not apply).  Synchronous; allocates and frees
+// device memory.
+int32_t mgpuBenchTuneMatmulEx(int32_t dtype, int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t act,
+                              int32_t hasResidual, float *libraryUs, float *mfmaUs) {
+  using mgpu::DType;
+  if (libraryUs) *libraryUs = 0.0f;
+  if (mfmaUs) *mfmaUs = 0.0f;
+  if (dtype < 0 || dtype > 2 || M <= 0 || N <= 0 || K <= 0 || act < 0 || act > 2 || (act && hasResidual)) return -1;
+  const DType dt = static_cast<DType>(dtype);
+  const size_t eb = dt == DType::F32 ? 4 : 2;
+  const hipDataType t = dt == DType::F32 ? HIP_R_32F : dt == DType::F16 ? HIP_R_16F : HIP_R_16BF;
+  Scratch x;
+  const bool ready = hipMalloc(&x.in, (size_t)M * K * eb) == hipSuccess && hipMalloc(&x.w, (size_t)K * N * eb) == hipSuccess &&
+                     hipMalloc(&x.out, (size_t)M * N * eb) == hipSuccess && hipMalloc(&x.bias, (size_t)N * eb) == hipSuccess &&
+                     hipMalloc(&x.workspace, kWorkspace) == hipSuccess && hipStreamCreate(&x.s) == hipSuccess &&
+                     hipEventCreate(&x.e0) == hipSuccess && hipEventCreate(&x.e1) == hipSuccess &&
+                     hipblasLtCreate(&x.lt) == HIPBLAS_STATUS_SUCCESS;
+  if (!ready) return -1;
+  // 0x3c bytes: 1.06 as fp16, 0.0115 as fp32, finite in every type
+  (void)hipMemsetAsync(x.in, 0x3c, (size_t)M * K * eb, x.s);
+  (void)hipMemsetAsync(x.w, 0x3c, (size_t)K * N * eb, x.s);
+  (void)hipMemsetAsync(x.out, 0x3c, (size_t)M * N * eb, x.s);
+  (void)hipMemsetAsync(x.bias, 0x3c, (size_t)N * eb, x.s);
+
+  // the descriptors mgpuMatmulEx builds: column-major view of the row-major operands
+  if (hipblasLtMatmulDescCreate(&x.op, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return -1;
+  hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_DEFAULT;
+  const bool relu = act == 1;
+  if (hasBias && relu) epilogue = HIPBLASLT_EPILOGUE_RELU_BIAS;
+  else if (hasBias) epilogue = HIPBLASLT_EPILOGUE_BIAS;
+  else if (relu) epilogue = HIPBLASLT_EPILOGUE_RELU;
+  (void)hipblasLtMatmulDescSetAttribute(x.op, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue));
+  if (hasBias) {
+    const int32_t biasType = (int32_t)t;
+    (void)hipblasLtMatmulDescSetAttribute(x.op, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &biasType, sizeof(biasType));
+    (void)hipblasLtMatmulDescSetAttribute(x.op, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &x.bias, sizeof(x.bias));
+  }
+  if (hipblasLtMatrixLayoutCreate(&x.a, t, N, K, N) != HIPBLAS_STATUS_SUCCESS ||
+      hipblasLtMatrixLayoutCreate(&x.b, t, K, M, K) != HIPBLAS_STATUS_SUCCESS ||
+      hipblasLtMatrixLayoutCreate(&x.d, t, N, M, N) != HIPBLAS_STATUS_SUCCESS)
+    return -1;
+  hipblasLtMatmulPreference_t pref = nullptr;
+  if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return -1;
+  const uint64_t ws = kWorkspace;
+  (void)hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
+  hipblasLtMatmulHeuristicResult_t results[kCandidates] = {};
+  int returned = 0;
+  const hipblasStatus_t st =
+      hipblasLtMatmulAlgoGetHeuristic(x.lt, x.op, x.a, x.b, x.d, x.d, pref, kCandidates, results, &returned);
+  hipblasLtMatmulPreferenceDestroy(pref);
+  if (st != HIPBLAS_STATUS_SUCCESS || returned == 0) return -1;
+
+  const float alpha = 1.0f, beta = hasResidual ? 1.0f : 0.0f;
+  auto libraryOnce = [&](int c) {
+    return hipblasLtMatmul(x.lt, x.op, &alpha, x.w, x.a, x.in, x.b, &beta, x.out, x.d, x.out, x.d, &results[c].algo,
+                           x.workspace, kWorkspace, x.s) == HIPBLAS_STATUS_SUCCESS;
+  };
+  // reps launches between two events after one untimed launch; milliseconds in total, < 0 on failure
+  auto timeLoop = [&](auto &&once, int reps) -> float {
+    try {
+      if (!once()) return -1.0f;
+      (void)hipEventRecord(x.e0, x.s);
+      for (int rep = 0; rep < reps; rep++)
+        if (!once()) return -1.0f;
+    } catch (const std::exception &) {
+      return -1.0f;
+    }
+    float ms = 0.0f;
+    if (hipEventRecord(x.e1, x.s) != hipSuccess || hipEventSynchronize(x.e1) != hipSuccess ||
+        hipEventElapsedTime(&ms, x.e0, x.e1) != hipSuccess)
+      return -1.0f;
+    return ms;
+  };
+  // Screening: three launches each; the kFinalists fastest go on to twenty launches each.
+  std::vector<std::pair<float, int>> screened;
+  for (int c = 0; c < returned; c++) {
+    if (results[c].state != HIPBLAS_STATUS_SUCCESS || results[c].workspaceSize > kWorkspace) continue;
+    const float ms = timeLoop([&] { return libraryOnce(c); }, 3);
+    if (ms >= 0.0f) screened.emplace_back(ms, c);
+  }
+  std::sort(screened.begin(), screened.end());
+  int best = -1;
+  float bestMs = -1.0f;
+  for (size_t i = 0; i < screened.size() && i < (size_t)kFinalists; i++) {
+    const float ms = timeLoop([&] { return libraryOnce(screened[i].second); }, 20);
+    if (ms >= 0.0f && (bestMs < 0.0f || ms < bestMs)) {
+      bestMs = ms;
+      best = screened[i].second;
+    }
+  }
+  if (best < 0) return -1;
+
+  auto libraryPath = [&] {
+    if (!libraryOnce(best)) return false;
+    if (act == 2) {
+      if (dt == DType::F16) mgpu::geluInPlaceF16(x.out, (size_t)M * N, x.s);
+      else if (dt == DType::BF16) mgpu::geluInPlaceBF16(x.out, (size_t)M * N, x.s);
+      else mgpu::geluInPlaceF32(static_cast<float *>(x.out), (size_t)M * N, x.s);
+    }
+    return true;
+  };
+  // The hand-written kernel on the same operands (`out` doubles as the residual).
+  const void *biasArg = hasBias ? x.bias : nullptr, *resArg = hasResidual ? x.out : nullptr;
+  const bool mfmaApplies = mgpu::gemmMfmaSupports(dt, x.in, x.w, biasArg, resArg, x.out, M, N, K);
+  auto mfmaPath = [&] {
+    mgpu::gemmMfma(dt, x.in, x.w, biasArg, resArg, x.out, M, N, K, act, x.s);
+    return true;
+  };
+  // Both paths in alternating runs of twenty launches, three runs each, so that they meet the
+  // same clocks: a lone burst of a kernel that has the device to itself for a millisecond runs
+  // faster than the same kernel in a layer.
+  float libraryMs = 0.0f, mfmaMs = 0.0f;
+  bool ok = true;
+  for (int round = 0; round < 3 && ok; round++) {
+    const float l = timeLoop(libraryPath, 20), m = mfmaApplies ? timeLoop(mfmaPath, 20) : 0.0f;
+    ok = l >= 0.0f && m >= 0.0f;
+    libraryMs += l;
+    mfmaMs += m;
+  }
+  (void)hipStreamSynchronize(x.s);
+  if (!ok) return -1;
+  if (libraryUs) *libraryUs = libraryMs * 1000.0f / 60.0f;
+  if (mfmaUs) *mfmaUs = mfmaMs * 1000.0f / 60.0f;
+  // three per cent of margin: a tie goes to the library
+  return mfmaApplies && mfmaMs < 0.97f * libraryMs ? 1 : 0;
+}
+
+} // extern "C"

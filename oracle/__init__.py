@@ -193,7 +193,7 @@ def qkv_bias_transpose(qkv, bias, bf16: bool = False):
 
 
 def decoding_context_layer(x, wqkv, wo, bo, w1, b1, w2, b2, heads: int, causal: bool = True,
-                           act: int = ACT_RELU):
+                           act: int = ACT_RELU, norm_first: bool = True):
     """All fp32 in, fp32 out: the signature of mgpuLLMDecodingContextLayer."""
     arrs = [_c(a, np.float32) for a in (x, wqkv, wo, bo, w1, b1, w2, b2)]
     B, S, d = x.shape
@@ -201,8 +201,8 @@ def decoding_context_layer(x, wqkv, wo, bo, w1, b1, w2, b2, heads: int, causal: 
     out = np.empty((B, S, d), np.float32)
     lib().oracle_decoding_context_layer(*[_p(a) for a in arrs], _p(out), ctypes.c_int64(B),
                                         ctypes.c_int64(S), ctypes.c_int64(d), ctypes.c_int64(ffn),
-                                        ctypes.c_int64(heads), ctypes.c_int(1 if causal else 0),
-                                        ctypes.c_int(act))
+                                        ctypes.c_int64(heads), ctypes.c_int(1 if norm_first else 0),
+                                        ctypes.c_int(1 if causal else 0), ctypes.c_int(act))
     return out
 
 

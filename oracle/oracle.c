@@ -447,6 +447,9 @@ static uint16_t *to_half_buf(const float *src, int64_t n) {
  * hard-wires 8 x 128 heads, causal, ReLU - LLM.cu:18-19,79-81,119-121) and
  * GEMMs accumulate in >= fp32 (the reference asks for fp16 accumulation,
  * Ops.cu:164-167, whose results only a CUDA run could pin).
+ * norm_first = 0 (declared by the reference, Ops.h:43-48, read by neither of its
+ * bodies; the meaning is the usual one of that flag) is the post-LN ordering of the
+ * same blocks: h = LN(x + proj(attention(x))), out = LN(h + ffn(h)), identity affine.
  * act: 1 ReLU, 2 GELU(erf).
  * pinned by: composition of the pinned pieces above; cross-checked against a
  * torch fp64 restatement in the tests.  Parity with the reference's own
@@ -455,7 +458,8 @@ ORACLE_API void oracle_decoding_context_layer(const float *input, const float *w
                                               const float *wo, const float *bo, const float *w1,
                                               const float *b1, const float *w2, const float *b2,
                                               float *output, int64_t B, int64_t S, int64_t d,
-                                              int64_t ffn, int64_t H, int causal, int act) {
+                                              int64_t ffn, int64_t H, int norm_first, int causal,
+                                              int act) {
   const int64_t M = B * S, Dh = d / H;
   uint16_t *xh = to_half_buf(input, M * d);
   uint16_t *wqkv_h = to_half_buf(wqkv, d * 3 * d);
@@ -466,21 +470,38 @@ ORACLE_API void oracle_decoding_context_layer(const float *input, const float *w
   float *t1 = (float *)malloc((size_t)M * 3 * d * sizeof(float));
   float *t2 = (float *)malloc((size_t)M * ffn * sizeof(float));
 
-  oracle_layernorm(xh, NULL, NULL, t0, 1e-5, M, d, 1);
-  uint16_t *a_h = to_half_buf(t0, M * d);
-  oracle_gemm(a_h, wqkv_h, NULL, NULL, t1, M, 3 * d, d, 0, 1);
-  uint16_t *qkv_h = to_half_buf(t1, M * 3 * d);
-  oracle_fmha(qkv_h, NULL, t0, B, S, H, Dh, 1.0 / sqrt((double)Dh), causal, 1);
-  uint16_t *ctx_h = to_half_buf(t0, M * d);
-  oracle_gemm(ctx_h, wo_h, bo_h, NULL, t0, M, d, d, 0, 1);
-  uint16_t *pr_h = to_half_buf(t0, M * d);
+  uint16_t *a_h = NULL, *qkv_h, *ctx_h, *pr_h, *y_h, *n2_h = NULL, *f_h;
   float *ysum = (float *)malloc((size_t)M * d * sizeof(float));
-  oracle_add_residual_layernorm(pr_h, xh, NULL, NULL, ysum, t0, 1e-5, M, d, 1);
-  uint16_t *y_h = to_half_buf(ysum, M * d);
-  uint16_t *n2_h = to_half_buf(t0, M * d);
-  oracle_gemm(n2_h, w1_h, b1_h, NULL, t2, M, ffn, d, act, 1);
-  uint16_t *f_h = to_half_buf(t2, M * ffn);
-  oracle_gemm(f_h, w2_h, b2_h, y_h, t0, M, d, ffn, 0, 1);
+  if (norm_first) { /* y = x + proj(attention(LN(x))), out = y + ffn(LN(y)) */
+    oracle_layernorm(xh, NULL, NULL, t0, 1e-5, M, d, 1);
+    a_h = to_half_buf(t0, M * d);
+    oracle_gemm(a_h, wqkv_h, NULL, NULL, t1, M, 3 * d, d, 0, 1);
+    qkv_h = to_half_buf(t1, M * 3 * d);
+    oracle_fmha(qkv_h, NULL, t0, B, S, H, Dh, 1.0 / sqrt((double)Dh), causal, 1);
+    ctx_h = to_half_buf(t0, M * d);
+    oracle_gemm(ctx_h, wo_h, bo_h, NULL, t0, M, d, d, 0, 1);
+    pr_h = to_half_buf(t0, M * d);
+    oracle_add_residual_layernorm(pr_h, xh, NULL, NULL, ysum, t0, 1e-5, M, d, 1);
+    y_h = to_half_buf(ysum, M * d);
+    n2_h = to_half_buf(t0, M * d);
+    oracle_gemm(n2_h, w1_h, b1_h, NULL, t2, M, ffn, d, act, 1);
+    f_h = to_half_buf(t2, M * ffn);
+    oracle_gemm(f_h, w2_h, b2_h, y_h, t0, M, d, ffn, 0, 1);
+  } else { /* post-LN: h = LN(x + proj(attention(x))), out = LN(h + ffn(h)) */
+    oracle_gemm(xh, wqkv_h, NULL, NULL, t1, M, 3 * d, d, 0, 1);
+    qkv_h = to_half_buf(t1, M * 3 * d);
+    oracle_fmha(qkv_h, NULL, t0, B, S, H, Dh, 1.0 / sqrt((double)Dh), causal, 1);
+    ctx_h = to_half_buf(t0, M * d);
+    oracle_gemm(ctx_h, wo_h, bo_h, NULL, t0, M, d, d, 0, 1);
+    pr_h = to_half_buf(t0, M * d);
+    oracle_add_residual_layernorm(pr_h, xh, NULL, NULL, ysum, t0, 1e-5, M, d, 1);
+    y_h = to_half_buf(t0, M * d); /* h, as stored */
+    oracle_gemm(y_h, w1_h, b1_h, NULL, t2, M, ffn, d, act, 1);
+    f_h = to_half_buf(t2, M * ffn);
+    oracle_gemm(f_h, w2_h, b2_h, NULL, t0, M, d, ffn, 0, 1);
+    n2_h = to_half_buf(t0, M * d);
+    oracle_add_residual_layernorm(n2_h, y_h, NULL, NULL, ysum, t0, 1e-5, M, d, 1);
+  }
   for (int64_t i = 0; i < M * d; i++)
     output[i] = half_bits_to_float(double_to_half_bits((double)t0[i]));
 

@@ -339,6 +339,10 @@ def test_cpu_runner_executes_the_layer_ops(tmp_path, oracle):
     ref = oracle.decoding_context_layer(x, *W, heads=H, causal=True, act=oracle.ACT_RELU)
     assert np.all(np.abs(got - ref) <= layer_tol(ref)), np.abs(got - ref).max()
     assert np.array_equal(got, got.astype(np.float16).astype(np.float32))  # the final cast comes from fp16
+    got, _ = run_cpu_plan(tmp_path, text.replace("norm_first = true", "norm_first = false"), [x] + W, np.float32,
+                          (B, S, d))
+    ref = oracle.decoding_context_layer(x, *W, heads=H, causal=True, act=oracle.ACT_RELU, norm_first=False)
+    assert np.all(np.abs(got - ref) <= layer_tol(ref)), np.abs(got - ref).max()  # post-LN ordering
 
     h16 = lambda *s: (0.05 * rng.standard_normal(s)).astype(np.float16)
     gam = lambda: (1 + 0.05 * rng.standard_normal(d)).astype(np.float16)

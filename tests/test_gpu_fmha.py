@@ -382,8 +382,9 @@ def test_fmha_cu_seqlens_packed_rows(pkg, gpu, oracle, rng, lens, max_s, causal,
 
 
 def test_fmha_profile_entry_point_matches_the_product_kernel(pkg, gpu):
-    """mgpuFusedMHAF16Profile is the head_dim-64 kernel with clock stamps: the same
-    output bits as mgpuFusedMHAF16, one record of ten counters per block, stamps in order."""
+    """mgpuBenchFusedMHAF16Profile (the benchmark's launch-loop library, not the kernel library) is the
+    head_dim-64 kernel with clock stamps: the same output bits as mgpuFusedMHAF16, one record of ten
+    counters per block, stamps in order."""
     import torch
     B, S, H, D = 2, 320, 3, 64
     g = torch.Generator(device=gpu).manual_seed(11)
@@ -392,10 +393,8 @@ def test_fmha_profile_entry_point_matches_the_product_kernel(pkg, gpu):
     out = torch.zeros_like(want)
     blocks = B * H * ((S + 127) // 128)
     stamps = torch.zeros(blocks * 10, dtype=torch.int64, device=gpu)
-    lib = pkg.ops()
-    got = lib.mgpuFusedMHAF16Profile(qkv.data_ptr(), out.data_ptr(), B, S, H, D ** -0.5, stamps.data_ptr(),
-                                     torch.cuda.current_stream().cuda_stream)
-    assert lib.mgpuOpsTakeLastError() is None
+    got = pkg.bench_loops().mgpuBenchFusedMHAF16Profile(qkv.data_ptr(), out.data_ptr(), B, S, H, D ** -0.5,
+                                                        stamps.data_ptr(), torch.cuda.current_stream().cuda_stream)
     assert got == blocks
     torch.cuda.synchronize()
     assert torch.equal(out, want)

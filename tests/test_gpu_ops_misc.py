@@ -179,3 +179,25 @@ def test_decoding_context_layer(pkg, gpu, oracle, rng, causal, relu, d, H):
     assert np.all(err <= layer_tol(ref)), err.max()
     # output is fp16-representable fp32, like the reference's final cast
     assert np.array_equal(got, got.astype(np.float16).astype(np.float32))
+
+
+@pytest.mark.parametrize("causal,relu,d,H", [(True, True, 512, 8), (False, False, 768, 12)])
+def test_decoding_context_layer_post_ln(pkg, gpu, oracle, rng, causal, relu, d, H):
+    """norm_first = false (Ops.h:43-48 declares the flag; the reference's bodies never read it): the post-LN
+    ordering, h = LN(x + proj(attention(x))), out = LN(h + ffn(h)).  The pre-LN result of the same
+    operands must differ, so a flag that is dropped on the way fails here."""
+    B, S, ffn = 4, 128, 2048
+    f = lambda *s, sc=0.03: (sc * rng.standard_normal(s)).astype(np.float32)
+    x = rng.standard_normal((B, S, d)).astype(np.float32)
+    W = [f(d, 3 * d), f(d, d), f(d), f(d, ffn), f(ffn), f(ffn, d), f(d)]
+    dev = [to_dev(w, gpu) for w in W]
+    got = pkg.decoding_context_layer(to_dev(x, gpu), *dev, heads=H, causal=causal, relu=relu,
+                                     norm_first=False).cpu().numpy()
+    act = oracle.ACT_RELU if relu else oracle.ACT_GELU
+    ref = oracle.decoding_context_layer(x, *W, heads=H, causal=causal, act=act, norm_first=False)
+    err = np.abs(got - ref)
+    assert np.all(err <= layer_tol(ref)), err.max()
+    assert err.mean() <= 5e-4
+    assert np.array_equal(got, got.astype(np.float16).astype(np.float32))
+    pre = pkg.decoding_context_layer(to_dev(x, gpu), *dev, heads=H, causal=causal, relu=relu).cpu().numpy()
+    assert np.abs(pre - got).max() > 0.1

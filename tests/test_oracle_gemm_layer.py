@@ -96,6 +96,27 @@ def test_decoding_context_layer_against_fp64_restatement(oracle, rng):
         assert np.abs(got - ref).max() < 2e-2 and np.abs(got - ref).mean() < 2e-3, (causal, act)
 
 
+def test_decoding_context_layer_post_ln_against_fp64_restatement(oracle, rng):
+    """norm_first = false: h = LN(x + proj(attention(x))), out = LN(h + ffn(h)), identity affine.  The fp64
+    restatement has no fp16 roundings; a pre-LN result, a missing residual or a LayerNorm in the wrong
+    place is off by far more than the bound."""
+    B, S, d, ffn, H = 2, 24, 128, 256, 2
+    f = lambda *s, sc=0.05: (sc * rng.standard_normal(s)).astype(np.float32)
+    x = rng.standard_normal((B, S, d)).astype(np.float32)
+    wqkv, wo, bo, w1, b1, w2, b2 = f(d, 3 * d), f(d, d), f(d), f(d, ffn), f(ffn), f(ffn, d), f(d)
+    for causal, act in [(True, oracle.ACT_RELU), (False, oracle.ACT_GELU)]:
+        got = oracle.decoding_context_layer(x, wqkv, wo, bo, w1, b1, w2, b2, heads=H, causal=causal, act=act,
+                                            norm_first=False)
+        X = x.astype(np.float64)
+        h1 = _ln(_attn(X @ wqkv, H, causal) @ wo + bo + X)
+        g = h1 @ w1 + b1
+        g = np.maximum(g, 0) if act == oracle.ACT_RELU else 0.5 * g * (1 + erf(g / np.sqrt(2)))
+        ref = _ln(g @ w2 + b2 + h1)
+        assert np.abs(got - ref).max() < 2e-2 and np.abs(got - ref).mean() < 2e-3, (causal, act)
+        pre = oracle.decoding_context_layer(x, wqkv, wo, bo, w1, b1, w2, b2, heads=H, causal=causal, act=act)
+        assert np.abs(pre - ref).max() > 0.1  # the two orderings are far apart on these operands
+
+
 def test_bert_layer_against_fp64_restatement(oracle, rng):
     B, S, d, ffn, H = 2, 20, 128, 256, 2
     h16 = lambda *s, sc=0.05: (sc * rng.standard_normal(s)).astype(np.float16)
