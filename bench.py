@@ -50,6 +50,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 MALL_BYTES = 256 << 20
+CACHE_MULTIPLE = 2.0  # footprint of the rotating buffer sets in units of the Infinity Cache (--cache-multiple)
 # HBM bytes per launch as counted by the hardware: profiles/hbm_traffic.json is
 # written from two rocprofv3 --pmc passes over this script (FETCH_SIZE, then
 # WRITE_SIZE, each scaled by what the same counter reads for the 64 MiB copy of
@@ -78,6 +79,10 @@ def parse_args():
     ap.add_argument("--repeats", type=int, default=7, help="timed regions of --steps launches each; the median is reported")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the copy / launch-floor / MFMA-loop probes")
+    ap.add_argument("--cache-multiple", type=float, default=2.0,
+                    help="total footprint of the rotating buffer sets of the cold measurements, in units of the 256 MiB "
+                         "Infinity Cache")
+    ap.add_argument("--no-runner", action="store_true", help="skip the end-to-end --rerun figures of the two runners")
     ap.add_argument("--tune-gemm", action="store_true",
                     help="measure the four GEMM shapes of the BERT-base layer with the tuner of the launch-loop library (library candidates "
                          "against the hand-written kernel) and print the lines of csrc/kernels/gemm_table.inc on stderr")
@@ -172,11 +177,15 @@ def device_info(torch) -> dict:
 
 
 def rotating_sets(bytes_per_set: int) -> int:
-    """Number of buffer sets whose total footprint exceeds the Infinity Cache."""
-    return max(2, (MALL_BYTES + bytes_per_set - 1) // bytes_per_set + 2)
+    """Number of buffer sets (bytes read + bytes written per launch each) whose total footprint is at
+    least twice the Infinity Cache: the launch loops walk them round robin without ever restarting, so
+    between two uses of a set the device moves a full rotation of other bytes."""
+    return max(3, int(CACHE_MULTIPLE * MALL_BYTES + bytes_per_set - 1) // bytes_per_set + 1)
 
 
-def hbm_entry(name, workload, dtype, bytes_per_launch, ms, steps, warm_ms=None):
+def hbm_entry(name, workload, dtype, bytes_per_launch, ms, steps, warm_ms=None, copy_us=None, copy_what=None):
+    """copy_us: microseconds per launch of the plain copy probe with the same bytes in and out (same number
+    of input streams, same rotation of buffer sets), timed in the same process right after the kernel."""
     us = ms * 1e3 / steps
     gbs = bytes_per_launch / us / 1e3
     e = {"name": name, "workload": workload, "dtype": dtype, "metric": "GB/s", "value": round(gbs, 1),
@@ -184,6 +193,11 @@ def hbm_entry(name, workload, dtype, bytes_per_launch, ms, steps, warm_ms=None):
          "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                       "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES.get(name)},
          "algorithmic_bytes": bytes_per_launch}
+    if copy_us:
+        e["copy_ceiling"] = {"us_per_launch": round(copy_us, 3), "GB/s": round(bytes_per_launch / copy_us / 1e3, 1),
+                             "what": copy_what}
+        e["copy_ceiling_GBs"] = e["copy_ceiling"]["GB/s"]
+        e["frac_of_copy_ceiling"] = round(copy_us / us, 4)
     if warm_ms is not None:
         wus = warm_ms * 1e3 / steps
         e["cache_resident"] = {"us_per_launch": round(wus, 3), "GB/s": round(bytes_per_launch / wus / 1e3, 1)}
@@ -286,6 +300,56 @@ def cpu_baselines(pkg, m, n, ln_bytes) -> dict:
     out["bert_layer"] = both(lambda: lib.mcpuBertEncoderLayerF16(P(xb), *[P(w) for w in W], None, P(ob), i64(B), i64(S), i64(d),
                                                                   i64(ffn), i64(H), ctypes.c_float(1e-5)),
                              4.0, 10, lambda s: s * 1e6, "us", "BERT-base encoder layer fp16 (32,128,768)")
+    return out
+
+
+def runner_end_to_end(pkg, reruns: int = 30) -> dict:
+    """The reference's own figure (tools/multi-device-gpu-runner/multi-device-gpu-runner.cpp:69-87: the model
+    run N times between two events, allocation, host-to-device and device-to-host copies of every run
+    included): this build's runners on the device plans of configs[0..2], host buffers pageable as the
+    reference's runner allocates them.  PCIe-inclusive, reported beside the kernel-only figures, never as
+    `value`."""
+    import re
+    import subprocess
+    import tempfile
+    P = os.path.dirname(os.path.abspath(pkg.__file__))
+    gpu_runner = os.path.join(P, "bin", "multi-device-gpu-runner")
+    cpu_runner = os.path.join(P, "bin", "multi-device-cpu-runner")
+    if not (os.path.exists(gpu_runner) and os.path.exists(cpu_runner)):
+        return {"error": "runners are not built"}
+    rng = np.random.default_rng(20240)
+    out = {}
+    with tempfile.TemporaryDirectory() as tmp:
+        def dat(name, a):
+            path = os.path.join(tmp, name)
+            a.tofile(path)
+            return path
+        cases = {
+            "add_f32": ("add.plan", [dat("a.dat", rng.uniform(-1, 1, (3, 640, 640)).astype(np.float32)),
+                                     dat("b.dat", rng.uniform(-1, 1, (3, 640, 640)).astype(np.float32))], 3 * 4915200),
+            "layernorm_f32": ("layernorm.plan", [dat("x.dat", rng.standard_normal((32, 128, 768)).astype(np.float32)),
+                                                 dat("g.dat", np.ones(768, np.float32)), dat("be.dat", np.zeros(768, np.float32))],
+                              2 * 32 * 128 * 768 * 4),
+            "fmha_b32_s128": ("fmha.plan", [dat("qkv.dat", (rng.standard_normal((32, 128, 3, 12, 64)) / 8).astype(np.float16))],
+                              32 * 128 * 768 * 2 * 4),
+        }
+        for name, (plan, files, nbytes) in cases.items():
+            entry = {"plan": f"plans/{plan}", "reruns": reruns, "bytes_over_pcie_per_run": nbytes}
+            for which, cmd in (("gpu_runner", [gpu_runner, os.path.join(P, "plans", plan), "--ops", os.path.join(pkg.LIB_DIR, "ops.hsaco")]),
+                               ("cpu_runner", [cpu_runner, os.path.join(P, "plans", plan)])):
+                n = reruns if which == "gpu_runner" or name != "fmha_b32_s128" else 3
+                try:
+                    r = subprocess.run(cmd + ["--data", ",".join(files), "--rerun", str(n)], capture_output=True, text=True,
+                                       timeout=120)
+                    m = re.search(r"Average time:\s*([0-9.eE+-]+)\s*seconds", r.stdout)
+                    entry[which + "_us_per_run"] = round(float(m.group(1)) * 1e6, 1) if (r.returncode == 0 and m) else None
+                except Exception as exc:  # a missing runner or a timeout: say so, the kernel figures stand
+                    entry[which + "_us_per_run"] = None
+                    entry[which + "_error"] = str(exc)[:200]
+            out[name] = entry
+    out["what"] = ("multi-device-gpu-runner / multi-device-cpu-runner <plan> --data ... --rerun N: seconds per run of the "
+                   "whole model call, device allocation, host-to-device and device-to-host copies included (pageable host "
+                   "buffers), as the reference's runner reports it")
     return out
 
 
@@ -476,6 +540,8 @@ def measure_ceilings(torch, loops, dev, gen, sp, ptrs, repeats) -> dict:
 
 def main():
     args = parse_args()
+    global CACHE_MULTIPLE
+    CACHE_MULTIPLE = max(1.0, args.cache_multiple)
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus must be 1 (multi-GPU runs are not part of it)",
               file=sys.stderr)
@@ -560,12 +626,15 @@ def main():
         ln_args = (ctypes.c_void_p(gamma.data_ptr()), ctypes.c_void_p(beta.data_ptr()), ctypes.c_float(1e-5), m, n)
         ms_cold = loop_ms(lambda: loops.mgpuBenchLayerNormF32(ptrs(xs), ptrs(ys), nsets, *ln_args, K, W, sp))
         ms_warm = loop_ms(lambda: loops.mgpuBenchLayerNormF32(ptrs(xs[:1]), ptrs(ys[:1]), 1, *ln_args, K, W, sp))
+        copy_ms = loop_ms(lambda: loops.mgpuProbeCopy(ptrs(xs), ptrs(ys), nsets, ctypes.c_size_t(m * n * 4), K, W, sp))
     else:
         ms_cold = timer.run(ln32, K, W, R)
         ms_warm = timer.run(lambda i: ln32(0), K, W, R)
     check()
+    COPY_WHAT = ("plain copy kernel (one 16-byte vector per lane, non-temporal stores) over the same buffer sets: as "
+                 "many bytes in and out, same rotation")
     headline = hbm_entry("layernorm_f32", "LayerNorm fp32 (32,128,768) eps=1e-5 [configs[1]]", "f32",
-                         ln_bytes, ms_cold, K, ms_warm)
+                         ln_bytes, ms_cold, K, ms_warm, copy_ms * 1e3 / K if loops else None, COPY_WHAT)
     del xs, ys, slab
 
     # ---------------- LayerNorm fp16 ------------------------------------------
@@ -586,12 +655,13 @@ def main():
             a16 = (ctypes.c_void_p(gh.data_ptr()), ctypes.c_void_p(bh.data_ptr()), ctypes.c_float(1e-5), m, n)
             ms = loop_ms(lambda: loops.mgpuBenchLayerNormF16(ptrs(xh), ptrs(yh), nsets, *a16, K, W, sp))
             msw = loop_ms(lambda: loops.mgpuBenchLayerNormF16(ptrs(xh[:1]), ptrs(yh[:1]), 1, *a16, K, W, sp))
+            copy_ms = loop_ms(lambda: loops.mgpuProbeCopy(ptrs(xh), ptrs(yh), nsets, ctypes.c_size_t(m * n * 2), K, W, sp))
         else:
             ms = timer.run(ln16, K, W, R)
             msw = timer.run(lambda i: ln16(0), K, W, R)
         check()
         kernels.append(hbm_entry("layernorm_f16", "LayerNorm fp16 (32,128,768)", "f16",
-                                 2 * m * n * 2 + 2 * n * 2, ms, K, msw))
+                                 2 * m * n * 2 + 2 * n * 2, ms, K, msw, copy_ms * 1e3 / K if loops else None, COPY_WHAT))
         del xh, yh, slab
 
     # ---------------- add fp32 (3,640,640) -------------------------------------
@@ -611,11 +681,16 @@ def main():
             torch.cuda.synchronize()
             ms = loop_ms(lambda: loops.mgpuBenchAddF32(ptrs(aa), ptrs(bb), ptrs(cc), nsets, ctypes.c_int64(ne), K, W, sp))
             msw = loop_ms(lambda: loops.mgpuBenchAddF32(ptrs(aa[:1]), ptrs(bb[:1]), ptrs(cc[:1]), 1, ctypes.c_int64(ne), K, W, sp))
+            copy_ms = loop_ms(lambda: loops.mgpuProbeCombine(ptrs(aa), ptrs(bb), ptrs(cc), nsets, ctypes.c_size_t(ne * 4),
+                                                             K, W, sp))
         else:
             ms = timer.run(add, K, W, R)
             msw = timer.run(lambda i: add(0), K, W, R)
         check()
-        kernels.append(hbm_entry("add_f32", "add fp32 (3,640,640) [configs[0]]", "f32", 3 * ne * 4, ms, K, msw))
+        kernels.append(hbm_entry("add_f32", "add fp32 (3,640,640) [configs[0]]", "f32", 3 * ne * 4, ms, K, msw,
+                                 copy_ms * 1e3 / K if loops else None,
+                                 "two-streams-in one-out probe (xor of two 16-byte vectors per lane, non-temporal store) "
+                                 "over the same buffer sets"))
         del aa, bb, cc, slab
 
     # ---------------- the same two kernels where launch latency is amortised ----
@@ -627,9 +702,10 @@ def main():
         yl = torch.empty_like(xl)
         torch.cuda.synchronize()
         ms = loop_ms(lambda: loops.mgpuBenchLayerNormF32(ptrs([xl]), ptrs([yl]), 1, *ln_args[:3], mL, n, 20, 3, sp))
+        copy_ms = loop_ms(lambda: loops.mgpuProbeCopy(ptrs([xl]), ptrs([yl]), 1, ctypes.c_size_t(mL * n * 4), 20, 3, sp))
         check()
         kernels.append(hbm_entry("layernorm_f32_large", f"LayerNorm fp32 ({mL},{n})", "f32",
-                                 2 * mL * n * 4 + 2 * n * 4, ms, 20))
+                                 2 * mL * n * 4 + 2 * n * 4, ms, 20, None, copy_ms * 1e3 / 20, COPY_WHAT))
         del xl, yl
     if want("layernorm_f32_wide") and loops:
         # a wide row (an LLM hidden size): one 256-thread block holds the row in registers
@@ -642,9 +718,10 @@ def main():
         torch.cuda.synchronize()
         ms = loop_ms(lambda: loops.mgpuBenchLayerNormF32(ptrs(xw), ptrs(yw), nsW, ctypes.c_void_p(gw.data_ptr()),
                                                          ctypes.c_void_p(bw.data_ptr()), ctypes.c_float(1e-5), mW, nW, 50, 5, sp))
+        copy_ms = loop_ms(lambda: loops.mgpuProbeCopy(ptrs(xw), ptrs(yw), nsW, ctypes.c_size_t(mW * nW * 4), 50, 5, sp))
         check()
         kernels.append(hbm_entry("layernorm_f32_wide", f"LayerNorm fp32 ({mW},{nW})", "f32",
-                                 2 * mW * nW * 4 + 2 * nW * 4, ms, 50))
+                                 2 * mW * nW * 4 + 2 * nW * 4, ms, 50, None, copy_ms * 1e3 / 50, COPY_WHAT))
         del xw, yw
     if want("add_f32_large") and loops:
         nl = 1 << 28
@@ -652,8 +729,10 @@ def main():
         cl = torch.empty_like(al)
         torch.cuda.synchronize()
         ms = loop_ms(lambda: loops.mgpuBenchAddF32(ptrs([al]), ptrs([bl]), ptrs([cl]), 1, ctypes.c_int64(nl), 20, 3, sp))
+        copy_ms = loop_ms(lambda: loops.mgpuProbeCombine(ptrs([al]), ptrs([bl]), ptrs([cl]), 1, ctypes.c_size_t(nl * 4), 20, 3, sp))
         check()
-        kernels.append(hbm_entry("add_f32_large", f"add fp32 ({nl} elements)", "f32", 3 * nl * 4, ms, 20))
+        kernels.append(hbm_entry("add_f32_large", f"add fp32 ({nl} elements)", "f32", 3 * nl * 4, ms, 20, None,
+                                 copy_ms * 1e3 / 20, "two-streams-in one-out probe over the same buffers"))
         del al, bl, cl
 
     # ---------------- fused MHA -------------------------------------------------
@@ -896,6 +975,30 @@ def main():
             if key and key in cpu_all:
                 e["cpu_baseline"] = cpu_all[key]
 
+    runner = None if args.no_runner else runner_end_to_end(pkg)
+
+    # The figures the north star names, gathered once more as the LAST keys of the line so that a
+    # reader who keeps only the tail of it still has them.
+    def star(e, flops=False):
+        if e is None:
+            return None
+        r = {"us_per_launch": e["us_per_launch"], e["metric"]: e["value"], "frac_of_peak": e["roofline"]["frac"]}
+        if "frac_of_copy_ceiling" in e:
+            r["copy_ceiling_GBs"] = e["copy_ceiling_GBs"]
+            r["frac_of_copy_ceiling"] = e["frac_of_copy_ceiling"]
+        if "cache_resident" in e:
+            r["cache_resident_us_per_launch"] = e["cache_resident"]["us_per_launch"]
+        if "hbm_frac" in e:
+            r["hbm_frac"] = e["hbm_frac"]
+        return r
+    by_name = {e["name"]: e for e in kernels}
+    north_star = {"layernorm_f32": star(headline), "layernorm_f16": star(by_name.get("layernorm_f16")),
+                  "add_f32": star(by_name.get("add_f32")), "fmha_b32_s512": star(by_name.get("fmha_b32_s512")),
+                  "fmha_b32_s128": star(by_name.get("fmha_b32_s128")),
+                  "fmha_b8_s512_masked": star(by_name.get("fmha_b8_s512_masked")),
+                  "bert_layer_us": by_name["bert_layer"]["value"] if "bert_layer" in by_name else None,
+                  "peaks": {"hbm_GBs": HBM_PEAK_GBS, "mfma_f16_TFLOPs": MFMA_F16_PEAK_TFLOPS}}
+
     result = {
         "metric": "LayerNorm GB/s (fp32 (32,128,768)); fMHA TFLOP/s and BERT-base layer us under 'kernels'",
         "value": headline["value"], "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -906,10 +1009,13 @@ def main():
                                    "direct ctypes launches" if args.no_graph else "hipGraph of K ctypes launches"),
                    "buffer_sets": rotating_sets(2 * m * n * 4)},
         "repeats": R, "roofline": headline["roofline"], "cache_resident": headline.get("cache_resident"),
+        "copy_ceiling": headline.get("copy_ceiling"), "frac_of_copy_ceiling": headline.get("frac_of_copy_ceiling"),
         "traffic_counted_at_commit": TRAFFIC_COMMIT,
         "cpu_baseline": cpu, "ceilings": ceilings, "fmha_phases": phases, "kernels": kernels,
+        "runner_end_to_end": runner,
         "device": torch.cuda.get_device_name(0),
         "device_info": device_info(torch),
+        "north_star": north_star,
     }
     print(json.dumps(result))
 

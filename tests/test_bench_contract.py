@@ -38,5 +38,12 @@ def test_one_json_line_with_the_contract_keys():
     assert abs(d["value"] - roof["achieved"]) < 1e-6
     cpu = d["cpu_baseline"]
     assert cpu["kind"] in ("port", "reference") and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
+    # the north star's figures are the last key of the line, each with the copy ceiling measured beside it
+    assert list(d)[-1] == "north_star"
+    for name in ("layernorm_f32", "add_f32"):
+        e = d["north_star"][name]
+        assert e["us_per_launch"] > 0 and 0 < e["frac_of_peak"] < 1 and e["copy_ceiling_GBs"] > 0
+        assert 0.3 < e["frac_of_copy_ceiling"] < 2.0
+    assert d["runner_end_to_end"]["add_f32"]["gpu_runner_us_per_run"] > 0
     # value = algorithmic bytes of one step over the measured time of one step
     assert abs(d["value"] - 25171968 / (d["ms_per_step"] * 1e-3) / 1e9) / d["value"] < 2e-3

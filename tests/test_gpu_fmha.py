@@ -423,6 +423,8 @@ def test_fmha_profile_entry_point_matches_the_product_kernel(pkg, gpu):
     (160, 2, 64, 2, None, False, "bf16"),
     (136, 1, 65, 1, None, False, "f16"),        # the first size past the 128-wide geometry
     (248, 1, 129, 2, [129], True, "f16"),       # one chunk short of the 256-wide geometry
+    (80, 16, 384, 22, None, True, "f16"),       # 704 causal work items: query blocks in pairs, head size 80 inside 128
+    (96, 32, 300, 8, None, True, "bf16"),       # 512 paired items with a middle block (3 query blocks), ragged last tile
 ])
 def test_fmha_other_head_sizes(pkg, gpu, oracle, rng, D, B, S, H, lens, causal, dtype):
     """Head sizes between the tile geometries (64, 128, 256) run inside the next larger one: rows in
