@@ -3,9 +3,10 @@
 // Replaces the kernel the reference's pipeline generates for onnx.Add
 // (1200 blocks x 1024 threads, one scalar element per thread:
 // include/multi-device-model-compiler/Dialect/Device/Transform/Passes.td:86-89)
-// with 128-bit loads and stores, several independent loads in flight per lane
-// and a grid sized to the machine.  One IEEE add per element: bit exact with
-// examples/add.ll:42-66.
+// with 128-bit loads and non-temporal 128-bit stores, one vector per lane and one
+// block per 256 vectors (the grid is sized to the array, not to the machine: blocks
+// are dispatched in index order, so the device sweeps one window of memory at a time).
+// One IEEE add per element: bit exact with examples/add.ll:42-66.
 #include "common.hpp"
 #include "mgpu_ops_internal.hpp"
 

@@ -61,7 +61,7 @@
 //     overlap, where add, fma, max3 and the f16 converts overlap completely
 //     and v_exp_f32 costs about 2;
 //   * accumulators stay in VGPRs (no AGPR copies);
-//   * three wavefronts share a SIMD (142 VGPRs) and are left to drift apart, so
+//   * three wavefronts share a SIMD (145 VGPRs) and are left to drift apart, so
 //     that one is in an MFMA phase while another does its softmax; s_setprio
 //     lets the MFMA phases win the issue slot.
 // The output tile is transposed through LDS so that every store instruction
@@ -77,7 +77,7 @@ namespace fmha_detail {
 
 // Geometry per head dimension D (64, 128 or 256).  At D = 64 a K or V tile is 8 KiB
 // (64 keys of 128 bytes, 8 MFMAs for the scores and 8 for P.V), the ring has three
-// stages and three blocks share a CU (146 VGPRs, three wavefronts per SIMD).  At
+// stages and three blocks share a CU (145 VGPRs, three wavefronts per SIMD).  At
 // D = 128 and 256 a tile is 16 KiB (64 keys of 256 bytes or 32 of 512: 16 + 16 MFMAs
 // per tile, half as many barriers and bursts of tile loads per MFMA) and the ring has
 // two stages, so that two blocks share a CU's LDS; accumulators and Q operands (64 + 32
