@@ -3,7 +3,7 @@
 
 A "step" is one pass of the hot path over one batch of synthetic input, with
 all inputs already resident in HBM when the timed region starts.  The headline
-workload is the LayerNorm configuration of BASELINE.json (configs[1]:
+workload is the LayerNorm configuration of the benchmark definition (configs[1]:
 fp32 (32,128,768), eps 1e-5); the other configurations (add, fp16 LayerNorm,
 fused MHA at three shapes, the BERT-base layer) are measured in the same run
 and reported under "kernels" in the same JSON line, each against the roofline

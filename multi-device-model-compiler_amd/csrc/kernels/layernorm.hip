@@ -113,7 +113,10 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
       }
     }
     const float var = group_sum<LANES>(sq) * inv_n;
-    const float rstd = 1.0f / sqrtf(var + eps);
+    // v_rsq_f32 (1 ulp) in place of the correctly rounded sqrt and division, two dependent
+    // sequences of a dozen instructions in the middle of the wavefront's one chain: fp16
+    // (4096, 768) 3.93 -> 3.80 us, (262144, 768) fp32 266 -> 263.5 us, the fp32 headline unchanged.
+    const float rstd = __builtin_amdgcn_rsqf(var + eps);
 
     u32x4 *yv = reinterpret_cast<u32x4 *>(normed + (size_t)row * n);
     u32x4 *sv = (RESIDUAL && sumOut) ? reinterpret_cast<u32x4 *>(sumOut + (size_t)row * n) : nullptr;
@@ -229,7 +232,7 @@ __global__ __launch_bounds__(256) void layernorm_cast_rows_kernel(const float *_
       }
     }
     const float var = group_sum<LANES>(sq) * inv_n;
-    const float rstd = 1.0f / sqrtf(var + eps);
+    const float rstd = __builtin_amdgcn_rsqf(var + eps);
 
     u32x4 *yv = reinterpret_cast<u32x4 *>(normed + (size_t)row * n);
 #pragma unroll
@@ -345,7 +348,7 @@ __global__ __launch_bounds__(256) void layernorm_block_kernel(
 #pragma unroll
     for (int r = 0; r < ROWS; r++) {
       const float var = (partial[1][r][0] + partial[1][r][1] + partial[1][r][2] + partial[1][r][3]) * inv_n;
-      rstd[r] = 1.0f / sqrtf(var + eps);
+      rstd[r] = __builtin_amdgcn_rsqf(var + eps);
     }
 
 #pragma unroll
@@ -409,7 +412,7 @@ __global__ __launch_bounds__(256) void layernorm_general_kernel(
     if (threadIdx.x % 64 == 0) partial[wave] = sq;
     __syncthreads();
     const float var = (partial[0] + partial[1] + partial[2] + partial[3]) * inv_n;
-    const float rstd = 1.0f / sqrtf(var + eps);
+    const float rstd = __builtin_amdgcn_rsqf(var + eps);
     for (int i = threadIdx.x; i < n; i += 256) {
       float v = value(i);
       if (RESIDUAL) {
