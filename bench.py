@@ -811,6 +811,28 @@ def main():
     # separate GELU pass where there is one) and the hand-written MFMA kernel the committed table names for the
     # shape; mgpuGemmMfmaF16 is the hand-written kernel by itself.  With --tune-gemm the shape is first measured
     # on this device (mgpuBenchTuneMatmulEx of the launch-loop library) and the table line that measurement gives is printed.
+    def tune_shape(M_, N_, K_, has_bias, act, residual):
+        """Measure one shape on this device and print the line of gemm_table.inc that the measurement gives."""
+        lib_us, mfma_us, best_us = ctypes.c_float(0), ctypes.c_float(0), ctypes.c_float(0)
+        index, version = ctypes.c_int32(-1), ctypes.c_int32(0)
+        kept = int(pkg.bench_loops().mgpuBenchTuneMatmulEx(1, M_, N_, K_, has_bias, act, residual,
+                                                           ctypes.byref(lib_us), ctypes.byref(mfma_us),
+                                                           ctypes.byref(best_us), ctypes.byref(index),
+                                                           ctypes.byref(version)))
+        if kept < 0:
+            raise RuntimeError("mgpuBenchTuneMatmulEx failed")
+        print(f"{{1, {M_}, {N_}, {K_}, {has_bias}, {act}, {residual}, {kept}}},  // library {lib_us.value:.1f} us "
+              f"(the best of its 64 answers {best_us.value:.1f}: solution {index.value} of hipBLASLt {version.value}), "
+              f"hand-written {mfma_us.value:.1f} us", file=sys.stderr)
+        return kept
+
+    if args.tune_gemm and want("decoding_layer"):
+        # the four GEMMs of the decoding layer below (4096 tokens, d_model 2048, feed-forward 2048)
+        tune_shape(4096, 6144, 2048, 0, 0, 0)
+        tune_shape(4096, 2048, 2048, 1, 0, 0)
+        tune_shape(4096, 2048, 2048, 1, 1, 0)
+        tune_shape(4096, 2048, 2048, 1, 0, 1)
+
     def gemm_case(name, workload, M_, K_, N_, act, residual):
         x = torch.randn((M_, K_), device=dev, generator=gen).half()
         wt = (0.02 * torch.randn((K_, N_), device=dev, generator=gen)).half()
@@ -829,15 +851,7 @@ def main():
             check()
             return ms * 1e3 / steps
 
-        tuned = None
-        if args.tune_gemm:
-            lib_us, mfma_us = ctypes.c_float(0), ctypes.c_float(0)
-            tuned = int(pkg.bench_loops().mgpuBenchTuneMatmulEx(1, M_, N_, K_, 1, act, int(residual),
-                                                                ctypes.byref(lib_us), ctypes.byref(mfma_us)))
-            if tuned < 0:
-                raise RuntimeError("mgpuBenchTuneMatmulEx failed")
-            print(f"{{1, {M_}, {N_}, {K_}, 1, {act}, {int(residual)}, {tuned}}},  // library {lib_us.value:.1f} us, "
-                  f"hand-written {mfma_us.value:.1f} us", file=sys.stderr)
+        tuned = tune_shape(M_, N_, K_, 1, act, int(residual)) if args.tune_gemm else None
         us_auto, us_mfma = gemm(lib.mgpuMatmulExF16), gemm(lib.mgpuGemmMfmaF16)
         flop = 2.0 * M_ * N_ * K_
         kernels.append({"name": name, "workload": workload,
@@ -923,12 +937,20 @@ def main():
         steps = max(10, K // 10)
         ms = Timer(torch, use_graph=False).run(dec, steps, 3, R)
         check()
+        lib.mgpuLLMOpsCacheWeights(1)   # the weights cast to fp16 once instead of on every call
+        try:
+            dec(0)
+            us_cached = Timer(torch, use_graph=False).run(dec, steps, 3, R) * 1e3 / steps
+        finally:
+            lib.mgpuLLMOpsCacheWeights(0)
+        check()
         us = ms * 1e3 / steps
         flop = 2.0 * B * S * d * (3 * d + d + 2 * ffn) + 4.0 * B * H * (d // H) * (S * (S + 1) / 2)
         kernels.append({"name": "decoding_layer",
                         "workload": "mgpuLLMDecodingContextLayer fp32 in/out (8,512,2048), 16 heads of 128, ffn 2048, "
                                     "causal, ReLU; fp32 weights cast to fp16 on every call, as in the reference",
                         "dtype": "f16", "metric": "us", "value": round(us, 1), "higher_is_better": False,
+                        "us_per_call_with_weight_cache": round(us_cached, 1),
                         "roofline": {"bound": "mfma", "achieved": round(flop / us / 1e6, 1),
                                      "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                      "frac": round(flop / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},

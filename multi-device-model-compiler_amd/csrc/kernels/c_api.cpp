@@ -45,6 +45,9 @@ void gpuLLMOpsInit() {
   mgpu::noAllocInit();
 }
 void gpuLLMOpsDeinit() { mgpu::llmDeinit(); }
+extern "C" void mgpuLLMOpsCacheWeights(int32_t enable) {
+  guarded([&] { mgpu::llmCacheWeights(enable != 0); });
+}
 
 void gpuOpsInit() {
   mgpu::gemmInit();

@@ -77,6 +77,28 @@ StreamState &sideOf(hipStream_t s) {
   return st;
 }
 
+// Opt-in cache of the reference layer's weights in fp16 (mgpuLLMOpsCacheWeights).  The layer's
+// ABI hands it fp32 weights and the reference casts all of them on every call (LLM.cu:55-57,
+// 84-90,100-106,124-130): 300 MB of HBM traffic per call at d_model 2048, on a side stream, next
+// to the GEMMs.  With the cache on, an array is cast the first time its (address, length) is seen
+// and the fp16 copy is kept until the cache is switched off or gpuLLMOpsDeinit; the caller
+// promises not to change a cached array in place.  Off by default: per-call casts, as in the
+// reference.  Guarded by scratchMutex.
+bool weightCacheOn = false;
+struct CachedWeight {
+  void *half = nullptr;
+  hipEvent_t ready = nullptr; // recorded behind the cast that filled the copy
+};
+std::map<std::pair<const float *, int64_t>, CachedWeight> weightCache;
+
+void dropWeightCache() { // scratchMutex held; the device idle or the copies no longer in use
+  for (auto &kv : weightCache) {
+    if (kv.second.half) (void)hipFree(kv.second.half);
+    if (kv.second.ready) (void)hipEventDestroy(kv.second.ready);
+  }
+  weightCache.clear();
+}
+
 // gamma = 1, beta = 0 in fp16 for the reference layer's LayerNorms, one pair
 // per model width, written once and kept until gpuLLMOpsDeinit.
 struct Identity {
@@ -165,7 +187,18 @@ void llmDeinit() {
     if (kv.second.beta) (void)hipFree(kv.second.beta);
   }
   identityOf.clear();
+  dropWeightCache();
+  weightCacheOn = false;
   initialised = false;
+}
+
+void llmCacheWeights(bool enable) {
+  std::lock_guard<std::mutex> lock(scratchMutex);
+  if (!enable && !weightCache.empty()) {
+    (void)hipDeviceSynchronize(); // a layer in flight may still read the copies
+    dropWeightCache();
+  }
+  weightCacheOn = enable;
 }
 
 void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *gemm_bias,
@@ -216,20 +249,61 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
     forkEvent = st.forkEvent;
     for (int i = 0; i < kCopyEvents; i++) copyEvent[i] = st.copyEvent[i];
   }
-  MGPU_CHECK_HIP(hipEventRecord(forkEvent, stream));
-  MGPU_CHECK_HIP(hipStreamWaitEvent(copyStream, forkEvent, 0));
-  castF32ToF16(arena.at(oWqkv), qkv, d * 3 * d, copyStream);
-  MGPU_CHECK_HIP(hipEventRecord(copyEvent[0], copyStream));
-  castF32ToF16(arena.at(oWo), gemm_weight, d * d, copyStream);
-  castF32ToF16(arena.at(oBo), gemm_bias, d, copyStream);
-  MGPU_CHECK_HIP(hipEventRecord(copyEvent[1], copyStream));
-  castF32ToF16(arena.at(oW1), ffn1_weight, d * ffn, copyStream);
-  castF32ToF16(arena.at(oB1), ffn1_bias, ffn, copyStream);
-  MGPU_CHECK_HIP(hipEventRecord(copyEvent[2], copyStream));
-  castF32ToF16(arena.at(oW2), ffn2_weight, ffn * d, copyStream);
-  castF32ToF16(arena.at(oB2), ffn2_bias, d, copyStream);
-  MGPU_CHECK_HIP(hipEventRecord(copyEvent[3], copyStream));
-  auto join = [&](int group) { MGPU_CHECK_HIP(hipStreamWaitEvent(stream, copyEvent[group], 0)); };
+  // The seven weight and bias arrays in fp16: cast by the side stream now, or - with the weight
+  // cache on - taken from the cache (cast once, when first seen, on the side stream as well).
+  struct Operand {
+    const float *src;
+    int64_t elems;
+    size_t slot;  // where the per-call copy goes in the arena
+    int group;    // the GEMM (0..3) that reads it
+    void *half;   // the fp16 copy the GEMM is given
+  };
+  Operand ops[7] = {{qkv, d * 3 * d, oWqkv, 0, nullptr},       {gemm_weight, d * d, oWo, 1, nullptr},
+                    {gemm_bias, d, oBo, 1, nullptr},           {ffn1_weight, d * ffn, oW1, 2, nullptr},
+                    {ffn1_bias, ffn, oB1, 2, nullptr},         {ffn2_weight, ffn * d, oW2, 3, nullptr},
+                    {ffn2_bias, d, oB2, 3, nullptr}};
+  bool forked = false, sideWork[kCopyEvents] = {false, false, false, false};
+  hipEvent_t cachedReady[7] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+  auto fork = [&] {
+    if (forked) return;
+    MGPU_CHECK_HIP(hipEventRecord(forkEvent, stream));
+    MGPU_CHECK_HIP(hipStreamWaitEvent(copyStream, forkEvent, 0));
+    forked = true;
+  };
+  {
+    std::lock_guard<std::mutex> lock(scratchMutex);
+    const bool useCache = weightCacheOn && !isCapturing(stream); // a capture neither allocates nor reads the cache's events
+    for (int i = 0; i < 7; i++) {
+      Operand &op = ops[i];
+      if (useCache) {
+        CachedWeight &cw = weightCache[{op.src, op.elems}];
+        if (!cw.half) { // first sight of this array: cast it once into memory of its own
+          MGPU_CHECK_HIP(hipMalloc(&cw.half, (size_t)op.elems * 2));
+          MGPU_CHECK_HIP(hipEventCreateWithFlags(&cw.ready, hipEventDisableTiming));
+          fork();
+          castF32ToF16(cw.half, op.src, op.elems, copyStream);
+          MGPU_CHECK_HIP(hipEventRecord(cw.ready, copyStream));
+        }
+        op.half = cw.half;
+        cachedReady[i] = cw.ready; // (an event long complete costs the stream nothing)
+      } else {
+        fork();
+        op.half = arena.at(op.slot);
+        castF32ToF16(op.half, op.src, op.elems, copyStream);
+        sideWork[op.group] = true;
+      }
+      // the casts go out in the order the GEMMs run; a group's event sits right behind its last cast
+      if ((i == 6 || ops[i + 1].group != op.group) && sideWork[op.group])
+        MGPU_CHECK_HIP(hipEventRecord(copyEvent[op.group], copyStream));
+    }
+  }
+  auto join = [&](int group) {
+    if (sideWork[group]) MGPU_CHECK_HIP(hipStreamWaitEvent(stream, copyEvent[group], 0));
+    for (int i = 0; i < 7; i++)
+      if (ops[i].group == group && cachedReady[i]) MGPU_CHECK_HIP(hipStreamWaitEvent(stream, cachedReady[i], 0));
+  };
+  const void *wqkvH = ops[0].half, *woH = ops[1].half, *boH = ops[2].half, *w1H = ops[3].half, *b1H = ops[4].half,
+             *w2H = ops[5].half, *b2H = ops[6].half;
 
   const void *gamma = arena.at(oGamma), *beta = arena.at(oBeta);
   if (const Identity *id = identityAffine(d, stream)) {
@@ -250,7 +324,7 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
     }
 
     join(0);
-    matmulEx(DType::F16, arena.at(oLn), arena.at(oWqkv), nullptr, arena.at(oQkv), nullptr, M, 3 * d,
+    matmulEx(DType::F16, arena.at(oLn), wqkvH, nullptr, arena.at(oQkv), nullptr, M, 3 * d,
              d, false, ACT_NONE, false, stream);
 
     // Attention context overwrites the first LayerNorm output, like the reference.
@@ -258,18 +332,18 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
              (int)heads, (int)(d_model / heads), 1.0f / sqrtf((float)(d_model / heads)), causal, stream);
 
     join(1);
-    matmulEx(DType::F16, arena.at(oLn), arena.at(oWo), arena.at(oBo), arena.at(oProj), nullptr, M, d,
+    matmulEx(DType::F16, arena.at(oLn), woH, boH, arena.at(oProj), nullptr, M, d,
              d, true, ACT_NONE, false, stream);
 
     layerNorm(DType::F16, arena.at(oProj), arena.at(oX), gamma, beta, arena.at(oY), arena.at(oLn), 1e-5f, (int)M,
               (int)d, stream);
 
     join(2);
-    matmulEx(DType::F16, arena.at(oLn), arena.at(oW1), arena.at(oB1), arena.at(oF), nullptr, M, ffn,
+    matmulEx(DType::F16, arena.at(oLn), w1H, b1H, arena.at(oF), nullptr, M, ffn,
              d, true, relu ? ACT_RELU : ACT_GELU, false, stream);
 
     join(3); // also the join of the fork: nothing of this call is left on the side stream after it
-    matmulEx(DType::F16, arena.at(oF), arena.at(oW2), arena.at(oB2), arena.at(oOut), arena.at(oY), M,
+    matmulEx(DType::F16, arena.at(oF), w2H, b2H, arena.at(oOut), arena.at(oY), M,
              d, ffn, true, ACT_NONE, true, stream);
   } else {
     // norm_first = false, the post-LN ordering of the same blocks (the reference declares the
@@ -278,21 +352,21 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
     // pre-LN ones, every intermediate stored in fp16 where the pre-LN path stores it.
     castF32ToF16(arena.at(oX), input, M * d, stream);
     join(0);
-    matmulEx(DType::F16, arena.at(oX), arena.at(oWqkv), nullptr, arena.at(oQkv), nullptr, M, 3 * d,
+    matmulEx(DType::F16, arena.at(oX), wqkvH, nullptr, arena.at(oQkv), nullptr, M, 3 * d,
              d, false, ACT_NONE, false, stream);
     fusedMHA(DType::F16, arena.at(oQkv), nullptr, arena.at(oLn), (int)batch, (int)seq_len,
              (int)heads, (int)(d_model / heads), 1.0f / sqrtf((float)(d_model / heads)), causal, stream);
     join(1);
-    matmulEx(DType::F16, arena.at(oLn), arena.at(oWo), arena.at(oBo), arena.at(oProj), nullptr, M, d,
+    matmulEx(DType::F16, arena.at(oLn), woH, boH, arena.at(oProj), nullptr, M, d,
              d, true, ACT_NONE, false, stream);
     // h (in oY) = LN(proj + x); the rounded sum is not needed again
     layerNorm(DType::F16, arena.at(oProj), arena.at(oX), gamma, beta, nullptr, arena.at(oY), 1e-5f, (int)M,
               (int)d, stream);
     join(2);
-    matmulEx(DType::F16, arena.at(oY), arena.at(oW1), arena.at(oB1), arena.at(oF), nullptr, M, ffn,
+    matmulEx(DType::F16, arena.at(oY), w1H, b1H, arena.at(oF), nullptr, M, ffn,
              d, true, relu ? ACT_RELU : ACT_GELU, false, stream);
     join(3);
-    matmulEx(DType::F16, arena.at(oF), arena.at(oW2), arena.at(oB2), arena.at(oProj), nullptr, M,
+    matmulEx(DType::F16, arena.at(oF), w2H, b2H, arena.at(oProj), nullptr, M,
              d, ffn, true, ACT_NONE, false, stream);
     layerNorm(DType::F16, arena.at(oProj), arena.at(oY), gamma, beta, nullptr, arena.at(oOut), 1e-5f, (int)M,
               (int)d, stream);

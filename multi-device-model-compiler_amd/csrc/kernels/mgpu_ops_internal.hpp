@@ -70,6 +70,8 @@ void pool2d(const float *input, float *output, int64_t N, int64_t C, int64_t H, 
 
 void llmInit();
 void llmDeinit();
+// Opt-in fp16 cache of the reference layer's fp32 weights (see llm.cpp); false also drops the copies.
+void llmCacheWeights(bool enable);
 void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *gemm_bias,
                           float *ffn1_weight, float *ffn1_bias, float *ffn2_weight,
                           float *ffn2_bias, float *output, int64_t batch, int64_t seq_len,

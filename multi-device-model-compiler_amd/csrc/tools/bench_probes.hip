@@ -26,8 +26,10 @@
 // Measurement plumbing only: nothing here is part of the kernel library.
 #include "bench_timed.hpp"
 
+#include <hip/hip_bf16.h>
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdint>
 
 namespace {
@@ -370,9 +372,36 @@ __global__ __launch_bounds__(256) void probe_lds_read_kernel(uint32_t *__restric
 
 using mgpu_bench::timed;
 
+// Element i becomes a hashed value spread evenly over (-amplitude, amplitude).
+template <typename T>
+__global__ void fill_varied_kernel(T *p, size_t n, float amplitude, uint32_t seed) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    uint32_t r = ((uint32_t)i + seed) * 2654435761u;
+    r ^= r >> 15;
+    r *= 0x85ebca6bu;
+    r ^= r >> 13;
+    p[i] = (T)(((float)(r >> 8) - 8388608.0f) * (amplitude / 8388608.0f));
+  }
+}
+
 } // namespace
 
 extern "C" {
+
+// Fills n elements (dtype 0 fp32, 1 fp16, 2 bf16) with values that differ from element to element,
+// spread over (-amplitude, amplitude).  What a timed matrix kernel should be fed: on a repeated
+// constant the device draws less power and clocks 10-40 % higher than on real data, by an amount
+// that differs from kernel to kernel.  Returns 0, or -1 on a launch error or an unknown dtype.
+int mgpuProbeFillVaried(void *p, size_t n, int dtype, float amplitude, unsigned seed, void *stream) {
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned blocks = (unsigned)std::min<size_t>((n + 255) / 256, 4096);
+  if (n == 0) return 0;
+  if (dtype == 0) fill_varied_kernel<float><<<blocks, 256, 0, s>>>((float *)p, n, amplitude, seed);
+  else if (dtype == 1) fill_varied_kernel<_Float16><<<blocks, 256, 0, s>>>((_Float16 *)p, n, amplitude, seed);
+  else if (dtype == 2) fill_varied_kernel<__hip_bfloat16><<<blocks, 256, 0, s>>>((__hip_bfloat16 *)p, n, amplitude, seed);
+  else return -1;
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
 
 // Milliseconds for `steps` copies of `bytes` (a multiple of 16) from src[i % nsets] to dst[i % nsets].
 float mgpuProbeCopy(void *const *src, void *const *dst, int nsets, size_t bytes, int steps, int warmup, void *stream) {

@@ -182,12 +182,16 @@ def test_tuner_measures_outside_the_kernel_library(pkg, gpu):
     M, K, N = 256, 160, 384
     loops = pkg.bench_loops()
     lib_us, mfma_us = ctypes.c_float(0), ctypes.c_float(0)
-    kept = loops.mgpuBenchTuneMatmulEx(1, M, N, K, 1, 0, 1, ctypes.byref(lib_us), ctypes.byref(mfma_us))
+    best_us, index, version = ctypes.c_float(0), ctypes.c_int32(-2), ctypes.c_int32(0)
+    kept = loops.mgpuBenchTuneMatmulEx(1, M, N, K, 1, 0, 1, ctypes.byref(lib_us), ctypes.byref(mfma_us),
+                                       ctypes.byref(best_us), ctypes.byref(index), ctypes.byref(version))
     assert kept in (0, 1)
     assert lib_us.value > 0 and mfma_us.value > 0
+    assert 0 < best_us.value <= 1.1 * lib_us.value     # the best of the library's answers is no slower than its first
+    assert index.value >= 0 and version.value > 0      # which library kernel that was
     assert kept == (1 if mfma_us.value < 0.97 * lib_us.value else 0)
-    assert loops.mgpuBenchTuneMatmulEx(7, M, N, K, 1, 0, 1, None, None) == -1      # no such element type
-    assert loops.mgpuBenchTuneMatmulEx(1, M, N, K, 1, 2, 1, None, None) == -1      # activation with a residual
+    assert loops.mgpuBenchTuneMatmulEx(7, M, N, K, 1, 0, 1, None, None, None, None, None) == -1      # no such element type
+    assert loops.mgpuBenchTuneMatmulEx(1, M, N, K, 1, 2, 1, None, None, None, None, None) == -1      # activation with a residual
     assert not hasattr(pkg.ops(), "mgpuMatmulExTune")
 
 

@@ -181,6 +181,35 @@ def test_decoding_context_layer(pkg, gpu, oracle, rng, causal, relu, d, H):
     assert np.array_equal(got, got.astype(np.float16).astype(np.float32))
 
 
+def test_decoding_context_layer_weight_cache(pkg, gpu, oracle, rng):
+    """mgpuLLMOpsCacheWeights(1): the fp32 weights are cast once, when first seen, and later calls reuse the
+    fp16 copies - same bits as the per-call casts; switching the cache off and on again drops the copies, so
+    weights changed in place in between are picked up."""
+    import torch
+    B, S, d, ffn, H = 2, 128, 512, 1024, 8
+    f = lambda *s, sc=0.03: (sc * rng.standard_normal(s)).astype(np.float32)
+    x = to_dev(rng.standard_normal((B, S, d)).astype(np.float32), gpu)
+    W = [to_dev(w, gpu) for w in (f(d, 3 * d), f(d, d), f(d), f(d, ffn), f(ffn), f(ffn, d), f(d))]
+    lib = pkg.ops()
+    plain = pkg.decoding_context_layer(x, *W, heads=H).clone()
+    lib.mgpuLLMOpsCacheWeights(1)
+    try:
+        first = pkg.decoding_context_layer(x, *W, heads=H).clone()     # fills the cache
+        again = pkg.decoding_context_layer(x, *W, heads=H).clone()     # served from it
+        assert torch.equal(first, plain) and torch.equal(again, plain)
+        W[1].mul_(0.5)                                                 # in place: the cache does not see it
+        stale = pkg.decoding_context_layer(x, *W, heads=H).clone()
+        assert torch.equal(stale, plain)
+        lib.mgpuLLMOpsCacheWeights(0)
+        lib.mgpuLLMOpsCacheWeights(1)
+        fresh = pkg.decoding_context_layer(x, *W, heads=H).clone()
+    finally:
+        lib.mgpuLLMOpsCacheWeights(0)
+    want = pkg.decoding_context_layer(x, *W, heads=H)
+    assert torch.equal(fresh, want) and not torch.equal(fresh, plain)
+    assert lib.mgpuOpsTakeLastError() is None
+
+
 @pytest.mark.parametrize("causal,relu,d,H", [(True, True, 512, 8), (False, False, 768, 12)])
 def test_decoding_context_layer_post_ln(pkg, gpu, oracle, rng, causal, relu, d, H):
     """norm_first = false (Ops.h:43-48 declares the flag; the reference's bodies never read it): the post-LN
