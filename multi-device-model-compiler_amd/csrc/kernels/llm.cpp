@@ -276,14 +276,24 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
     for (int i = 0; i < 7; i++) {
       Operand &op = ops[i];
       if (useCache) {
-        CachedWeight &cw = weightCache[{op.src, op.elems}];
-        if (!cw.half) { // first sight of this array: cast it once into memory of its own
-          MGPU_CHECK_HIP(hipMalloc(&cw.half, (size_t)op.elems * 2));
-          MGPU_CHECK_HIP(hipEventCreateWithFlags(&cw.ready, hipEventDisableTiming));
-          fork();
-          castF32ToF16(cw.half, op.src, op.elems, copyStream);
-          MGPU_CHECK_HIP(hipEventRecord(cw.ready, copyStream));
+        const std::pair<const float *, int64_t> key{op.src, op.elems};
+        auto hit = weightCache.find(key);
+        if (hit == weightCache.end()) { // first sight of this array: cast it once into memory of its own
+          CachedWeight fresh;           // entered into the cache only once its cast is on the side stream
+          MGPU_CHECK_HIP(hipMalloc(&fresh.half, (size_t)op.elems * 2));
+          try {
+            MGPU_CHECK_HIP(hipEventCreateWithFlags(&fresh.ready, hipEventDisableTiming));
+            fork();
+            castF32ToF16(fresh.half, op.src, op.elems, copyStream);
+            MGPU_CHECK_HIP(hipEventRecord(fresh.ready, copyStream));
+          } catch (...) {
+            if (fresh.ready) (void)hipEventDestroy(fresh.ready);
+            (void)hipFree(fresh.half);
+            throw;
+          }
+          hit = weightCache.emplace(key, fresh).first;
         }
+        const CachedWeight &cw = hit->second;
         op.half = cw.half;
         cachedReady[i] = cw.ready; // (an event long complete costs the stream nothing)
       } else {
