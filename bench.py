@@ -813,17 +813,17 @@ def main():
     # on this device (mgpuBenchTuneMatmulEx of the launch-loop library) and the table line that measurement gives is printed.
     def tune_shape(M_, N_, K_, has_bias, act, residual):
         """Measure one shape on this device and print the line of gemm_table.inc that the measurement gives."""
-        lib_us, mfma_us, best_us = ctypes.c_float(0), ctypes.c_float(0), ctypes.c_float(0)
+        times = (ctypes.c_float * 4)()
         index, version = ctypes.c_int32(-1), ctypes.c_int32(0)
-        kept = int(pkg.bench_loops().mgpuBenchTuneMatmulEx(1, M_, N_, K_, has_bias, act, residual,
-                                                           ctypes.byref(lib_us), ctypes.byref(mfma_us),
-                                                           ctypes.byref(best_us), ctypes.byref(index),
-                                                           ctypes.byref(version)))
+        kept = int(pkg.bench_loops().mgpuBenchTuneMatmulEx(1, M_, N_, K_, has_bias, act, residual, times,
+                                                           ctypes.byref(index), ctypes.byref(version)))
         if kept < 0:
             raise RuntimeError("mgpuBenchTuneMatmulEx failed")
-        print(f"{{1, {M_}, {N_}, {K_}, {has_bias}, {act}, {residual}, {kept}}},  // library {lib_us.value:.1f} us "
-              f"(the best of its 64 answers {best_us.value:.1f}: solution {index.value} of hipBLASLt {version.value}), "
-              f"hand-written {mfma_us.value:.1f} us", file=sys.stderr)
+        print(f"{{1, {M_}, {N_}, {K_}, {has_bias}, {act}, {residual}, {kept & 1}, {kept >> 1}}},  // library "
+              f"{times[0]:.1f} us (the best of its 64 answers {times[3]:.1f}: solution {index.value} of hipBLASLt "
+              f"{version.value}), hand-written {times[1]:.1f} us, library on a K-major weight {times[2]:.1f} us",
+              file=sys.stderr)
+        kept &= 1
         return kept
 
     if args.tune_gemm and want("decoding_layer"):
@@ -891,7 +891,7 @@ def main():
                                         B, S, d, ffn, H, 1e-5, s)
 
         steps = max(10, K // 10)
-        us_no_alloc = None
+        us_no_alloc = us_cached = None
         if loops:
             # the calls come from a C++ loop, like a compiled model's: seven kernels per call
             layer(0)  # first use of the GEMM shapes, untimed
@@ -905,6 +905,15 @@ def main():
             loops.mgpuBenchBertEncoderLayerF16(*largs, 0, 200, 0, sp)
             ms = loop_ms(lambda: loops.mgpuBenchBertEncoderLayerF16(*largs, 0, steps, 3, sp))
             us_no_alloc = loop_ms(lambda: loops.mgpuBenchBertEncoderLayerF16(*largs, 1, steps, 3, sp)) * 1e3 / steps
+            # with the weight cache on, the GEMMs that the library runs fastest on a K-major weight get the
+            # cache's transposed copy
+            lib.mgpuLLMOpsCacheWeights(1)
+            try:
+                layer(0)
+                torch.cuda.synchronize()
+                us_cached = loop_ms(lambda: loops.mgpuBenchBertEncoderLayerF16(*largs, 0, steps, 3, sp)) * 1e3 / steps
+            finally:
+                lib.mgpuLLMOpsCacheWeights(0)
         else:
             ms = Timer(torch, use_graph=False).run(layer, steps, 3, R)
         check()
@@ -913,6 +922,7 @@ def main():
         kernels.append({"name": "bert_layer", "workload": "BERT-base encoder layer fp16 (32,128,768) [configs[4]]",
                         "dtype": "f16", "metric": "us", "value": round(us, 1), "higher_is_better": False,
                         "us_per_call_no_alloc_entry_point": us_no_alloc and round(us_no_alloc, 1),
+                        "us_per_call_with_weight_cache": us_cached and round(us_cached, 1),
                         "roofline": {"bound": "mfma", "achieved": round(flop / us / 1e6, 1),
                                      "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                      "frac": round(flop / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},

@@ -215,14 +215,18 @@ void mgpuLLMDecodingContextLayer(float *input, float *qkv, float *gemm_weight, f
                                  bool norm_first, bool is_casual, bool is_relu,
                                  mgpuStream_t stream);
 
-/* Opt-in cache of that layer's weights in fp16; no counterpart in the reference, which casts
- * all seven fp32 weight and bias arrays to fp16 on every call (LLM.cu:55-57,84-90,100-106,
- * 124-130: 300 MB of memory traffic per call at d_model 2048).  After
- * mgpuLLMOpsCacheWeights(1) an array is cast the first time its (address, length) is seen
- * and the fp16 copy is reused by every later call; the caller promises not to change a
- * cached array in place.  mgpuLLMOpsCacheWeights(0) waits for the device, frees the copies
- * and returns to per-call casts (the default).  Calls under stream capture always cast per
- * call.  The first call that meets a new array allocates (hipMalloc). */
+/* Opt-in cache of the layers' weights; no counterpart in the reference, which casts all seven
+ * fp32 weight and bias arrays of the layer above to fp16 on every call (LLM.cu:55-57,84-90,
+ * 100-106,124-130: 300 MB of memory traffic per call at d_model 2048).  After
+ * mgpuLLMOpsCacheWeights(1) an array is converted the first time its (address, shape) is seen
+ * and the copy is reused by every later call; the caller promises not to change a cached array
+ * in place.  The copies are fp16, and a weight matrix is kept transposed ([N, K], K contiguous)
+ * where the GEMM library multiplies that layout faster; mgpuBertEncoderLayerF16, whose weights
+ * are fp16 already, takes such transposed copies for the GEMMs that gain from them.  Results
+ * stay within the layers' tolerances but are not bit-identical to the uncached path (another
+ * GEMM kernel, another summation order).  mgpuLLMOpsCacheWeights(0) waits for the device, frees
+ * the copies and returns to the default.  Calls under stream capture never use the cache.  The
+ * first call that meets a new array allocates (hipMalloc) a copy of its size in fp16. */
 void mgpuLLMOpsCacheWeights(int32_t enable);
 
 /* Post-LN BERT encoder layer on fp16 tensors; no counterpart in the reference

@@ -158,7 +158,7 @@ def bench_loops() -> ctypes.CDLL:
         lib.mgpuBenchFusedMHAF16Profile.argtypes = [_c_void_p, _c_void_p] + [_c_int32] * 3 + [_c_float, _c_void_p,
                                                                                                _c_void_p]
         lib.mgpuBenchTuneMatmulEx.restype = _c_int32
-        lib.mgpuBenchTuneMatmulEx.argtypes = [_c_int32] + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p] * 5
+        lib.mgpuBenchTuneMatmulEx.argtypes = [_c_int32] + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p] * 3
         _bench = lib
     return _bench
 

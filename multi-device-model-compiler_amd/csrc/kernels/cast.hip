@@ -148,6 +148,23 @@ void castToF32(float *dst, const void *src, size_t size, hipStream_t stream, con
   }
 }
 
+
+// dst[c][r] = T(src[r][c]) for a row-major rows x cols matrix: 64 x 64 tiles through LDS (one
+// padding column against bank conflicts), coalesced on both sides.  Runs once per weight array
+// (the weight cache of the layers), so it is written for clarity, not for the last GB/s.
+template <typename TO, typename TI>
+__global__ __launch_bounds__(256) void transpose_cast_kernel(TO *__restrict__ dst, const TI *__restrict__ src,
+                                                             int64_t rows, int64_t cols) {
+  __shared__ float tile[64][65];
+  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+  const int tx = threadIdx.x % 64, ty = threadIdx.x / 64;
+  for (int i = ty; i < 64; i += 4)
+    if (r0 + i < rows && c0 + tx < cols) tile[i][tx] = (float)src[(r0 + i) * cols + c0 + tx];
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4)
+    if (c0 + i < cols && r0 + tx < rows) dst[(c0 + i) * rows + r0 + tx] = (TO)tile[tx][i];
+}
+
 } // namespace
 
 void castF32ToF16(void *dst, const float *src, size_t size, hipStream_t stream) {
@@ -161,6 +178,24 @@ void castF32ToBF16(void *dst, const float *src, size_t size, hipStream_t stream)
 }
 void castBF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream) {
   castToF32<bf16_t>(dst, src, size, stream, "castBF16ToF32");
+}
+
+void transposeCastF32ToF16(void *dst, const float *src, int64_t rows, int64_t cols, hipStream_t stream) {
+  if (rows <= 0 || cols <= 0) return;
+  if (!dst || !src) fail("transposeCastF32ToF16: null pointer");
+  const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
+  if ((rows + 63) / 64 > 65535) fail("transposeCastF32ToF16: more than 4194240 rows");
+  transpose_cast_kernel<_Float16, float><<<grid, dim3(256), 0, stream>>>(static_cast<_Float16 *>(dst), src, rows, cols);
+  MGPU_CHECK_LAUNCH("transpose_cast_kernel");
+}
+void transposeF16(void *dst, const void *src, int64_t rows, int64_t cols, hipStream_t stream) {
+  if (rows <= 0 || cols <= 0) return;
+  if (!dst || !src) fail("transposeF16: null pointer");
+  const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
+  if ((rows + 63) / 64 > 65535) fail("transposeF16: more than 4194240 rows");
+  transpose_cast_kernel<_Float16, _Float16><<<grid, dim3(256), 0, stream>>>(static_cast<_Float16 *>(dst),
+                                                                        static_cast<const _Float16 *>(src), rows, cols);
+  MGPU_CHECK_LAUNCH("transpose_cast_kernel");
 }
 
 void fillF16(void *dst, size_t count, float value, hipStream_t stream) {

@@ -82,11 +82,13 @@ struct Plan {
   bool handWritten = false; // serve the shape with gemm_mfma.hip when the operands allow it
 };
 
-// Shapes decided offline: {type (1 fp16, 2 bf16), M, N, K, hasBias, act, hasResidual, hand-written kernel?}.
+// Shapes decided offline: {type (1 fp16, 2 bf16), M, N, K, hasBias, act, hasResidual, hand-written kernel
+// (against the library, both on the ABI's [K, N] weight)?, the library on a K-major copy of the weight
+// ahead of both?}.
 struct TableEntry {
   int dt;
   int64_t M, N, K;
-  int hasBias, act, hasResidual, handWritten;
+  int hasBias, act, hasResidual, handWritten, kMajorLibrary;
 };
 const TableEntry kTable[] = {
 #include "gemm_table.inc"
@@ -112,7 +114,19 @@ int forcedKernel() {
   return mode;
 }
 
-using Key = std::tuple<int64_t, int64_t, int64_t, int, int, int, int>;
+bool mfmaShape(DType dt, int64_t M, int64_t N, int64_t K) {
+  return (dt == DType::F16 || dt == DType::BF16) && M > 0 && M % 128 == 0 && (N % 128 == 0 || N % 96 == 0) && K % 32 == 0;
+}
+
+const TableEntry *tableRow(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual) {
+  for (const TableEntry &e : kTable)
+    if (e.dt == (int)dt && e.M == M && e.N == N && e.K == K && e.hasBias == (int)hasBias && e.act == act &&
+        e.hasResidual == (int)hasResidual)
+      return &e;
+  return nullptr;
+}
+
+using Key = std::tuple<int64_t, int64_t, int64_t, int, int, int, int, int>;
 std::map<Key, Plan> plans;
 
 hipDataType dataType(DType dt) {
@@ -139,9 +153,9 @@ constexpr int kCandidates = 16; // heuristic answers looked through for one that
 // Builds (once per shape, flags and type) the library's descriptors and picks its
 // algorithms; decides which kernel serves the shape.  No measurement, no allocation
 // beyond the library's host-side descriptors.
-Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual) {
+Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual, bool weightKMajor) {
   const bool relu = act == ACT_RELU;
-  const Key key{M, N, K, (int)hasBias, act, (int)hasResidual, (int)dt};
+  const Key key{M, N, K, (int)hasBias, act, (int)hasResidual, (int)dt, (int)weightKMajor};
   auto it = plans.find(key);
   if (it != plans.end()) return it->second;
 
@@ -162,9 +176,15 @@ Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, 
     MGPU_CHECK_BLAS(hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE,
                                                     &biasType, sizeof(biasType)));
   }
-  // Column-major view of the row-major operands: A = weight (N x K, ld N),
-  // B = input (K x M, ld K), C/D = output (N x M, ld N).
-  MGPU_CHECK_BLAS(hipblasLtMatrixLayoutCreate(&p.a, t, N, K, N));
+  // Column-major view of the row-major operands: A = weight (N x K, ld N; a K-major weight is
+  // the K x N matrix with ld K, transposed), B = input (K x M, ld K), C/D = output (N x M, ld N).
+  if (weightKMajor) {
+    const hipblasOperation_t transposed = HIPBLAS_OP_T;
+    MGPU_CHECK_BLAS(hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_TRANSA, &transposed, sizeof(transposed)));
+    MGPU_CHECK_BLAS(hipblasLtMatrixLayoutCreate(&p.a, t, K, N, K));
+  } else {
+    MGPU_CHECK_BLAS(hipblasLtMatrixLayoutCreate(&p.a, t, N, K, N));
+  }
   MGPU_CHECK_BLAS(hipblasLtMatrixLayoutCreate(&p.b, t, K, M, K));
   MGPU_CHECK_BLAS(hipblasLtMatrixLayoutCreate(&p.d, t, N, M, N));
 
@@ -191,14 +211,11 @@ Plan &getPlan(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, 
       p.hasNoWs = true;
     }
 
-  // The kernel: the table, else the rule; a measurement only when asked for.
-  const bool mfmaShape = (dt == DType::F16 || dt == DType::BF16) && M > 0 && M % 128 == 0 && (N % 128 == 0 || N % 96 == 0) && K % 32 == 0;
-  p.handWritten = mfmaShape && ruleSaysHandWritten(M, N, K, act);
-  for (const TableEntry &e : kTable)
-    if (e.dt == (int)dt && e.M == M && e.N == N && e.K == K && e.hasBias == (int)hasBias && e.act == act &&
-        e.hasResidual == (int)hasResidual)
-      p.handWritten = mfmaShape && e.handWritten != 0;
+  // The kernel: the table, else the rule.
+  p.handWritten = mfmaShape(dt, M, N, K) && ruleSaysHandWritten(M, N, K, act);
+  if (const TableEntry *e = tableRow(dt, M, N, K, hasBias, act, hasResidual)) p.handWritten = mfmaShape(dt, M, N, K) && e->handWritten != 0;
   if (forcedKernel()) p.handWritten = forcedKernel() == 2;
+  if (weightKMajor) p.handWritten = false; // the hand-written kernel reads [K, N] weights only
   return plans.emplace(key, p).first->second;
 }
 
@@ -220,9 +237,18 @@ void gemmDeinit() {
   ltHandle = nullptr;
 }
 
+bool gemmPrefersKMajor(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual) {
+  if (forcedKernel()) return forcedKernel() == 1;
+  if (const TableEntry *e = tableRow(dt, M, N, K, hasBias, act, hasResidual)) return e->kMajorLibrary != 0;
+  // Nobody measured the shape: the library's kernels for K-major weights were ahead of its
+  // kernels for [K, N] weights at every shape measured, so the copy pays wherever the library
+  // would serve the shape anyway.
+  return !(mfmaShape(dt, M, N, K) && ruleSaysHandWritten(M, N, K, act));
+}
+
 void matmulEx(DType dt, const void *input, const void *weight, const void *bias, void *output,
               const void *residual, int64_t M, int64_t N, int64_t K, bool hasBias, int act,
-              bool hasResidual, hipStream_t stream) {
+              bool hasResidual, hipStream_t stream, bool weightKMajor) {
   if (M < 0 || N < 0 || K < 0) fail("matmul: negative shape");
   if (M == 0 || N == 0) return;
   if (K == 0) fail("matmul: K must be positive");
@@ -235,7 +261,7 @@ void matmulEx(DType dt, const void *input, const void *weight, const void *bias,
     fail("matmul: an activation cannot be combined with a residual");
 
   std::lock_guard<std::mutex> lock(planMutex);
-  const Plan &p = getPlan(dt, M, N, K, hasBias, act, hasResidual);
+  const Plan &p = getPlan(dt, M, N, K, hasBias, act, hasResidual, weightKMajor);
   if (p.handWritten && gemmMfmaSupports(dt, input, weight, hasBias ? bias : nullptr,
                                         hasResidual ? residual : nullptr, output, M, N, K)) {
     gemmMfma(dt, input, weight, hasBias ? bias : nullptr, hasResidual ? residual : nullptr, output, M, N, K, act,

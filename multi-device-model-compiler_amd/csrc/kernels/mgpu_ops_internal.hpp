@@ -38,6 +38,9 @@ void castF32ToF16(void *dst, const float *src, size_t size, hipStream_t stream);
 void castF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream);
 void castF32ToBF16(void *dst, const float *src, size_t size, hipStream_t stream);
 void castBF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream);
+// dst[c][r] = src[r][c] of a row-major rows x cols matrix (fp32 -> fp16 / fp16 -> fp16)
+void transposeCastF32ToF16(void *dst, const float *src, int64_t rows, int64_t cols, hipStream_t stream);
+void transposeF16(void *dst, const void *src, int64_t rows, int64_t cols, hipStream_t stream);
 void fillF16(void *dst, size_t count, float value, hipStream_t stream);
 void fillI32(int32_t *dst, size_t count, int32_t value, hipStream_t stream);
 
@@ -49,9 +52,15 @@ void addFusedQKVBiasTransposeF16(void *q, void *k, void *v, void *qkv, const voi
 enum Activation { ACT_NONE = 0, ACT_RELU = 1, ACT_GELU = 2 };
 void gemmInit();
 void gemmDeinit();
+// weightKMajor: the weight is stored [N, K] (each output column's K values contiguous) instead of
+// the ABI's [K, N]; the layers' weight cache keeps such copies, which the library multiplies
+// faster.  Always served by the library.
 void matmulEx(DType dt, const void *input, const void *weight, const void *bias, void *output,
               const void *residual, int64_t M, int64_t N, int64_t K, bool hasBias, int act,
-              bool hasResidual, hipStream_t stream);
+              bool hasResidual, hipStream_t stream, bool weightKMajor = false);
+// Should a caller that can keep a K-major copy of the weight hand that one to matmulEx for this
+// problem?  (The committed table, else: wherever the library would serve the shape.)
+bool gemmPrefersKMajor(DType dt, int64_t M, int64_t N, int64_t K, bool hasBias, int act, bool hasResidual);
 
 // Hand-written MFMA GEMM (gemm_mfma.hip): fp16 / bf16, M a multiple of 128, N of
 // 128 or 96, K of 32, 16-byte aligned operands; bias and residual may be null.

@@ -1,8 +1,9 @@
-// The GEMM tuner behind `bench.py --tune-gemm`: for one shape and epilogue it times
-// hipBLASLt's candidate algorithms (the [K, N] row-major weight of mgpuMatmulEx, fp32
-// accumulation, bias / ReLU epilogue, a separate exact-erf GELU pass where there is one)
-// against the hand-written MFMA kernel, on scratch operands, its own stream and its own
-// workspace, and says which side won.  Its answers are the rows of
+// The GEMM tuner behind `bench.py --tune-gemm`: for one shape and epilogue it times the
+// three ways mgpuMatmulEx can run it - hipBLASLt on the [K, N] row-major weight of the ABI,
+// the hand-written MFMA kernel on the same weight, and hipBLASLt on a K-major ([N, K]) copy
+// of the weight, which the layers' weight cache can supply - with fp32 accumulation, bias /
+// ReLU epilogue and a separate exact-erf GELU pass where the library runs one, on scratch
+// operands, its own stream and its own workspace.  Its answers are the rows of
 // csrc/kernels/gemm_table.inc; the kernel library itself never measures.
 // Measurement plumbing only: nothing here is part of the kernel library.
 #include "mgpu_ops_internal.hpp"
@@ -17,24 +18,37 @@
 #include <utility>
 #include <vector>
 
+extern "C" int mgpuProbeFillVaried(void *p, size_t n, int dtype, float amplitude, unsigned seed, void *stream);
+
 namespace {
 
 constexpr size_t kWorkspace = 32u * 1024u * 1024u;
 constexpr int kCandidates = 64; // heuristic answers asked for and screened
 constexpr int kFinalists = 4;   // re-timed at length after the screening pass
 
+// The library's side of one weight layout: descriptors as mgpuMatmulEx builds them and the
+// heuristic's answers.
+struct LibraryProblem {
+  hipblasLtMatmulDesc_t op = nullptr;
+  hipblasLtMatrixLayout_t a = nullptr;
+  hipblasLtMatmulHeuristicResult_t results[kCandidates] = {};
+  int returned = 0;
+  int first = -1; // what mgpuMatmulEx runs: the first answer that fits the workspace
+  ~LibraryProblem() {
+    if (a) hipblasLtMatrixLayoutDestroy(a);
+    if (op) hipblasLtMatmulDescDestroy(op);
+  }
+};
+
 struct Scratch {
   void *in = nullptr, *w = nullptr, *out = nullptr, *res = nullptr, *bias = nullptr, *workspace = nullptr;
   hipStream_t s = nullptr;
   hipEvent_t e0 = nullptr, e1 = nullptr;
   hipblasLtHandle_t lt = nullptr;
-  hipblasLtMatmulDesc_t op = nullptr;
-  hipblasLtMatrixLayout_t a = nullptr, b = nullptr, d = nullptr;
+  hipblasLtMatrixLayout_t b = nullptr, d = nullptr;
   ~Scratch() {
     if (d) hipblasLtMatrixLayoutDestroy(d);
     if (b) hipblasLtMatrixLayoutDestroy(b);
-    if (a) hipblasLtMatrixLayoutDestroy(a);
-    if (op) hipblasLtMatmulDescDestroy(op);
     if (lt) hipblasLtDestroy(lt);
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
@@ -47,28 +61,24 @@ struct Scratch {
 
 } // namespace
 
-extern "C" int mgpuProbeFillVaried(void *p, size_t n, int dtype, float amplitude, unsigned seed, void *stream);
-
 extern "C" {
 
-// dtype: 0 fp32, 1 fp16, 2 bf16; act: 0 none, 1 ReLU, 2 GELU.  Compares the two kernels
-// mgpuMatmulEx chooses between - the library's first heuristic answer that fits the workspace
-// (plus the GELU pass) and the hand-written kernel - and returns 1 when the hand-written one is
-// faster by more than three per cent, 0 when the library is kept (also for shapes the
-// hand-written kernel does not take), -1 when nothing could be measured.  *libraryUs / *mfmaUs
-// receive their microseconds per launch (0 where the hand-written kernel does not apply).  For
-// information, the fastest of the library's 64 first answers is timed beside them:
-// *bestLibraryUs, and *solutionIndex / *libraryVersion, the library's own index of that kernel
-// and the hipBLASLt version the index belongs to.  Synchronous; allocates and frees device memory.
+// dtype: 0 fp32, 1 fp16, 2 bf16; act: 0 none, 1 ReLU, 2 GELU.  times[0..3] receive microseconds
+// per launch of: [0] the library's first heuristic answer that fits the workspace (plus the GELU
+// pass) on the [K, N] weight - what mgpuMatmulEx runs when the library serves the shape; [1] the
+// hand-written kernel (0 where it does not take the shape); [2] the library's first answer on a
+// K-major copy of the weight; [3] for information, the fastest of the library's 64 first answers
+// on the [K, N] weight, whose own index and hipBLASLt version go to *solutionIndex /
+// *libraryVersion.  Returns -1 when nothing could be measured, else bit 0: the hand-written
+// kernel beats [0] by more than three per cent (a tie goes to the library); bit 1: [2] beats the
+// better of [0] and [1] by more than three per cent (a caller that holds a K-major copy should
+// hand that one over).  Synchronous; allocates and frees device memory.
 int32_t mgpuBenchTuneMatmulEx(int32_t dtype, int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t act,
-                              int32_t hasResidual, float *libraryUs, float *mfmaUs, float *bestLibraryUs,
-                              int32_t *solutionIndex, int32_t *libraryVersion) {
-  if (bestLibraryUs) *bestLibraryUs = 0.0f;
+                              int32_t hasResidual, float *times, int32_t *solutionIndex, int32_t *libraryVersion) {
+  using mgpu::DType;
+  if (times) times[0] = times[1] = times[2] = times[3] = 0.0f;
   if (solutionIndex) *solutionIndex = -1;
   if (libraryVersion) *libraryVersion = 0;
-  using mgpu::DType;
-  if (libraryUs) *libraryUs = 0.0f;
-  if (mfmaUs) *mfmaUs = 0.0f;
   if (dtype < 0 || dtype > 2 || M <= 0 || N <= 0 || K <= 0 || act < 0 || act > 2 || (act && hasResidual)) return -1;
   const DType dt = static_cast<DType>(dtype);
   const size_t eb = dt == DType::F32 ? 4 : 2;
@@ -84,6 +94,7 @@ int32_t mgpuBenchTuneMatmulEx(int32_t dtype, int64_t M, int64_t N, int64_t K, in
   // Activations of unit variance and weights of standard deviation 0.02, every element different:
   // what a layer feeds these kernels.  On constant operands the device clocks 10-40 % higher, by a
   // different amount for each kernel, and the ranking measured there is not the one real data gives.
+  // (The same weight bytes serve as the [K, N] and as the K-major matrix: only time is measured.)
   if (mgpuProbeFillVaried(x.in, (size_t)M * K, dtype, 1.73f, 1u, x.s) != 0 ||
       mgpuProbeFillVaried(x.w, (size_t)K * N, dtype, 0.035f, 2u, x.s) != 0 ||
       mgpuProbeFillVaried(x.res, (size_t)M * N, dtype, 1.73f, 3u, x.s) != 0 ||
@@ -91,37 +102,54 @@ int32_t mgpuBenchTuneMatmulEx(int32_t dtype, int64_t M, int64_t N, int64_t K, in
     return -1;
 
   // the descriptors mgpuMatmulEx builds: column-major view of the row-major operands
-  if (hipblasLtMatmulDescCreate(&x.op, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return -1;
-  hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_DEFAULT;
-  const bool relu = act == 1;
-  if (hasBias && relu) epilogue = HIPBLASLT_EPILOGUE_RELU_BIAS;
-  else if (hasBias) epilogue = HIPBLASLT_EPILOGUE_BIAS;
-  else if (relu) epilogue = HIPBLASLT_EPILOGUE_RELU;
-  (void)hipblasLtMatmulDescSetAttribute(x.op, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue));
-  if (hasBias) {
-    const int32_t biasType = (int32_t)t;
-    (void)hipblasLtMatmulDescSetAttribute(x.op, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &biasType, sizeof(biasType));
-    (void)hipblasLtMatmulDescSetAttribute(x.op, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &x.bias, sizeof(x.bias));
-  }
-  if (hipblasLtMatrixLayoutCreate(&x.a, t, N, K, N) != HIPBLAS_STATUS_SUCCESS ||
-      hipblasLtMatrixLayoutCreate(&x.b, t, K, M, K) != HIPBLAS_STATUS_SUCCESS ||
+  if (hipblasLtMatrixLayoutCreate(&x.b, t, K, M, K) != HIPBLAS_STATUS_SUCCESS ||
       hipblasLtMatrixLayoutCreate(&x.d, t, N, M, N) != HIPBLAS_STATUS_SUCCESS)
     return -1;
-  hipblasLtMatmulPreference_t pref = nullptr;
-  if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return -1;
-  const uint64_t ws = kWorkspace;
-  (void)hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
-  hipblasLtMatmulHeuristicResult_t results[kCandidates] = {};
-  int returned = 0;
-  const hipblasStatus_t st =
-      hipblasLtMatmulAlgoGetHeuristic(x.lt, x.op, x.a, x.b, x.d, x.d, pref, kCandidates, results, &returned);
-  hipblasLtMatmulPreferenceDestroy(pref);
-  if (st != HIPBLAS_STATUS_SUCCESS || returned == 0) return -1;
+  auto describe = [&](LibraryProblem &p, bool kMajor) {
+    if (hipblasLtMatmulDescCreate(&p.op, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return false;
+    hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_DEFAULT;
+    const bool relu = act == 1;
+    if (hasBias && relu) epilogue = HIPBLASLT_EPILOGUE_RELU_BIAS;
+    else if (hasBias) epilogue = HIPBLASLT_EPILOGUE_BIAS;
+    else if (relu) epilogue = HIPBLASLT_EPILOGUE_RELU;
+    (void)hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue));
+    if (hasBias) {
+      const int32_t biasType = (int32_t)t;
+      (void)hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &biasType, sizeof(biasType));
+      (void)hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &x.bias, sizeof(x.bias));
+    }
+    if (kMajor) {
+      const hipblasOperation_t transposed = HIPBLAS_OP_T;
+      (void)hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_TRANSA, &transposed, sizeof(transposed));
+    }
+    if (hipblasLtMatrixLayoutCreate(&p.a, t, kMajor ? K : N, kMajor ? N : K, kMajor ? K : N) != HIPBLAS_STATUS_SUCCESS)
+      return false;
+    hipblasLtMatmulPreference_t pref = nullptr;
+    if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return false;
+    const uint64_t ws = kWorkspace;
+    (void)hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
+    const hipblasStatus_t st =
+        hipblasLtMatmulAlgoGetHeuristic(x.lt, p.op, p.a, x.b, x.d, x.d, pref, kCandidates, p.results, &p.returned);
+    hipblasLtMatmulPreferenceDestroy(pref);
+    if (st != HIPBLAS_STATUS_SUCCESS) return false;
+    for (int c = 0; c < p.returned && p.first < 0; c++)
+      if (p.results[c].state == HIPBLAS_STATUS_SUCCESS && p.results[c].workspaceSize <= kWorkspace) p.first = c;
+    return p.first >= 0;
+  };
+  LibraryProblem plain, kMajor;
+  if (!describe(plain, false) || !describe(kMajor, true)) return -1;
 
   const float alpha = 1.0f, beta = hasResidual ? 1.0f : 0.0f;
-  auto libraryOnce = [&](int c) {
-    return hipblasLtMatmul(x.lt, x.op, &alpha, x.w, x.a, x.in, x.b, &beta, hasResidual ? x.res : x.out, x.d, x.out, x.d, &results[c].algo,
-                           x.workspace, kWorkspace, x.s) == HIPBLAS_STATUS_SUCCESS;
+  auto libraryOnce = [&](const LibraryProblem &p, int c) {
+    if (hipblasLtMatmul(x.lt, p.op, &alpha, x.w, p.a, x.in, x.b, &beta, hasResidual ? x.res : x.out, x.d, x.out, x.d,
+                        &p.results[c].algo, x.workspace, kWorkspace, x.s) != HIPBLAS_STATUS_SUCCESS)
+      return false;
+    if (act == 2) {
+      if (dt == DType::F16) mgpu::geluInPlaceF16(x.out, (size_t)M * N, x.s);
+      else if (dt == DType::BF16) mgpu::geluInPlaceBF16(x.out, (size_t)M * N, x.s);
+      else mgpu::geluInPlaceF32(static_cast<float *>(x.out), (size_t)M * N, x.s);
+    }
+    return true;
   };
   // reps launches between two events after one untimed launch; milliseconds in total, < 0 on failure
   auto timeLoop = [&](auto &&once, int reps) -> float {
@@ -139,42 +167,30 @@ int32_t mgpuBenchTuneMatmulEx(int32_t dtype, int64_t M, int64_t N, int64_t K, in
       return -1.0f;
     return ms;
   };
-  // Screening: three launches each; the kFinalists fastest go on to twenty launches each.
+  // Screening of the [K, N] answers: three launches each; the kFinalists fastest go on to twenty.
   std::vector<std::pair<float, int>> screened;
-  for (int c = 0; c < returned; c++) {
-    if (results[c].state != HIPBLAS_STATUS_SUCCESS || results[c].workspaceSize > kWorkspace) continue;
-    const float ms = timeLoop([&] { return libraryOnce(c); }, 3);
+  for (int c = 0; c < plain.returned; c++) {
+    if (plain.results[c].state != HIPBLAS_STATUS_SUCCESS || plain.results[c].workspaceSize > kWorkspace) continue;
+    const float ms = timeLoop([&] { return libraryOnce(plain, c); }, 3);
     if (ms >= 0.0f) screened.emplace_back(ms, c);
   }
-  if (screened.empty()) return -1;
-  const int first = screened.front().second; // what mgpuMatmulEx runs: the first answer that fits the workspace
   std::sort(screened.begin(), screened.end());
   int best = -1;
   float bestMs = -1.0f;
   for (size_t i = 0; i < screened.size() && i < (size_t)kFinalists; i++) {
-    const float ms = timeLoop([&] { return libraryOnce(screened[i].second); }, 20);
+    const float ms = timeLoop([&] { return libraryOnce(plain, screened[i].second); }, 20);
     if (ms >= 0.0f && (bestMs < 0.0f || ms < bestMs)) {
       bestMs = ms;
       best = screened[i].second;
     }
   }
   if (best < 0) return -1;
-  if (solutionIndex) *solutionIndex = hipblaslt_ext::getIndexFromAlgo(results[best].algo);
+  if (solutionIndex) *solutionIndex = hipblaslt_ext::getIndexFromAlgo(plain.results[best].algo);
   if (libraryVersion) {
     int v = 0;
     if (hipblasLtGetVersion(x.lt, &v) == HIPBLAS_STATUS_SUCCESS) *libraryVersion = v;
   }
 
-  auto libraryPath = [&](int c) {
-    if (!libraryOnce(c)) return false;
-    if (act == 2) {
-      if (dt == DType::F16) mgpu::geluInPlaceF16(x.out, (size_t)M * N, x.s);
-      else if (dt == DType::BF16) mgpu::geluInPlaceBF16(x.out, (size_t)M * N, x.s);
-      else mgpu::geluInPlaceF32(static_cast<float *>(x.out), (size_t)M * N, x.s);
-    }
-    return true;
-  };
-  // The hand-written kernel on the same operands.
   const void *biasArg = hasBias ? x.bias : nullptr, *resArg = hasResidual ? x.res : nullptr;
   const bool mfmaApplies = mgpu::gemmMfmaSupports(dt, x.in, x.w, biasArg, resArg, x.out, M, N, K);
   auto mfmaPath = [&] {
@@ -184,24 +200,26 @@ int32_t mgpuBenchTuneMatmulEx(int32_t dtype, int64_t M, int64_t N, int64_t K, in
   // The paths in alternating runs of twenty launches, three runs each, so that they meet the
   // same clocks: a lone burst of a kernel that has the device to itself for a millisecond runs
   // faster than the same kernel in a layer.
-  float firstMs = 0.0f, bestRunMs = 0.0f, mfmaMs = 0.0f;
+  float ms[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   bool ok = true;
   for (int round = 0; round < 3 && ok; round++) {
-    const float f = timeLoop([&] { return libraryPath(first); }, 20);
-    const float b = best == first ? f : timeLoop([&] { return libraryPath(best); }, 20);
+    const float f = timeLoop([&] { return libraryOnce(plain, plain.first); }, 20);
     const float m = mfmaApplies ? timeLoop(mfmaPath, 20) : 0.0f;
-    ok = f >= 0.0f && b >= 0.0f && m >= 0.0f;
-    firstMs += f;
-    bestRunMs += b;
-    mfmaMs += m;
+    const float k = timeLoop([&] { return libraryOnce(kMajor, kMajor.first); }, 20);
+    const float b = best == plain.first ? f : timeLoop([&] { return libraryOnce(plain, best); }, 20);
+    ok = f >= 0.0f && m >= 0.0f && k >= 0.0f && b >= 0.0f;
+    ms[0] += f;
+    ms[1] += m;
+    ms[2] += k;
+    ms[3] += b;
   }
   (void)hipStreamSynchronize(x.s);
   if (!ok) return -1;
-  if (libraryUs) *libraryUs = firstMs * 1000.0f / 60.0f;
-  if (bestLibraryUs) *bestLibraryUs = bestRunMs * 1000.0f / 60.0f;
-  if (mfmaUs) *mfmaUs = mfmaMs * 1000.0f / 60.0f;
-  // against the library kernel the product would run; three per cent of margin: a tie goes to the library
-  return mfmaApplies && mfmaMs < 0.97f * firstMs ? 1 : 0;
+  if (times)
+    for (int i = 0; i < 4; i++) times[i] = ms[i] * 1000.0f / 60.0f;
+  const bool handWritten = mfmaApplies && ms[1] < 0.97f * ms[0];
+  const float bestOfAbi = handWritten ? ms[1] : ms[0];
+  return (handWritten ? 1 : 0) | (ms[2] < 0.97f * bestOfAbi ? 2 : 0);
 }
 
 } // extern "C"

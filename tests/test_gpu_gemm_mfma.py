@@ -175,23 +175,24 @@ def test_gemm_mfma_refuses_a_misaligned_bias(pkg, gpu):
 
 def test_tuner_measures_outside_the_kernel_library(pkg, gpu):
     """The tuner that writes gemm_table.inc lives with the benchmark's launch loops
-    (mgpuBenchTuneMatmulEx): it times the library's candidates against the hand-written kernel on
-    its own operands and reports both times; an unusable request reports -1; and the kernel
-    library exports no tuning entry point."""
+    (mgpuBenchTuneMatmulEx): it times the library on the ABI's [K, N] weight, the hand-written kernel and the
+    library on a K-major weight on its own operands and reports all three; an unusable request reports -1; and
+    the kernel library exports no tuning entry point."""
     import ctypes
     M, K, N = 256, 160, 384
     loops = pkg.bench_loops()
-    lib_us, mfma_us = ctypes.c_float(0), ctypes.c_float(0)
-    best_us, index, version = ctypes.c_float(0), ctypes.c_int32(-2), ctypes.c_int32(0)
-    kept = loops.mgpuBenchTuneMatmulEx(1, M, N, K, 1, 0, 1, ctypes.byref(lib_us), ctypes.byref(mfma_us),
-                                       ctypes.byref(best_us), ctypes.byref(index), ctypes.byref(version))
-    assert kept in (0, 1)
-    assert lib_us.value > 0 and mfma_us.value > 0
-    assert 0 < best_us.value <= 1.1 * lib_us.value     # the best of the library's answers is no slower than its first
+    times = (ctypes.c_float * 4)()
+    index, version = ctypes.c_int32(-2), ctypes.c_int32(0)
+    kept = loops.mgpuBenchTuneMatmulEx(1, M, N, K, 1, 0, 1, times, ctypes.byref(index), ctypes.byref(version))
+    assert 0 <= kept <= 3
+    library, mfma, k_major, best = list(times)
+    assert library > 0 and mfma > 0 and k_major > 0
+    assert 0 < best <= 1.1 * library                   # the best of the library's answers is no slower than its first
     assert index.value >= 0 and version.value > 0      # which library kernel that was
-    assert kept == (1 if mfma_us.value < 0.97 * lib_us.value else 0)
-    assert loops.mgpuBenchTuneMatmulEx(7, M, N, K, 1, 0, 1, None, None, None, None, None) == -1      # no such element type
-    assert loops.mgpuBenchTuneMatmulEx(1, M, N, K, 1, 2, 1, None, None, None, None, None) == -1      # activation with a residual
+    assert (kept & 1) == (1 if mfma < 0.97 * library else 0)
+    assert (kept >> 1) == (1 if k_major < 0.97 * min(library, mfma if kept & 1 else library) else 0)
+    assert loops.mgpuBenchTuneMatmulEx(7, M, N, K, 1, 0, 1, None, None, None) == -1      # no such element type
+    assert loops.mgpuBenchTuneMatmulEx(1, M, N, K, 1, 2, 1, None, None, None) == -1      # activation with a residual
     assert not hasattr(pkg.ops(), "mgpuMatmulExTune")
 
 

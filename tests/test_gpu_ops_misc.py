@@ -162,6 +162,34 @@ def test_bert_encoder_layer_config4(pkg, gpu, oracle):
         assert err.mean() <= 5e-4
 
 
+def test_bert_encoder_layer_weight_cache(pkg, gpu, oracle):
+    """With mgpuLLMOpsCacheWeights(1) the BERT layer hands the GEMMs the committed table marks (QKV and FFN2 at
+    configs[4]) a transposed copy of their weight, kept by the cache: same layer against the oracle, the same
+    bits on the second call, and an odd shape (nothing in the table, library everywhere) as well."""
+    import torch
+    rng = np.random.Generator(np.random.PCG64(20246))
+    lib = pkg.ops()
+    for B, S, d, ffn, H in ((32, 128, 768, 3072, 12), (3, 50, 192, 200, 3)):
+        h16 = lambda *s: (0.02 * rng.standard_normal(s)).astype(np.float16)
+        gam = lambda: (1 + 0.02 * rng.standard_normal(d)).astype(np.float16)
+        x = rng.standard_normal((B, S, d)).astype(np.float16)
+        P = [h16(d, 3 * d), h16(3 * d), h16(d, d), h16(d), gam(), h16(d), h16(d, ffn), h16(ffn), h16(ffn, d),
+             h16(d), gam(), h16(d)]
+        dev = [to_dev(p, gpu) for p in P]
+        ref = oracle.bert_layer_f16(x, *P, heads=H)
+        lib.mgpuLLMOpsCacheWeights(1)
+        try:
+            first = pkg.bert_encoder_layer(to_dev(x, gpu), *dev, heads=H).clone()
+            again = pkg.bert_encoder_layer(to_dev(x, gpu), *dev, heads=H).clone()
+        finally:
+            lib.mgpuLLMOpsCacheWeights(0)
+        assert torch.equal(first, again)
+        err = np.abs(first.cpu().numpy().astype(np.float32) - ref)
+        assert np.all(err <= layer_tol(ref)), err.max()
+        assert err.mean() <= 5e-4
+    assert lib.mgpuOpsTakeLastError() is None
+
+
 @pytest.mark.parametrize("causal,relu,d,H", [(True, True, 512, 8), (False, False, 512, 8), (True, True, 1024, 8),
                                              (True, False, 512, 2)])
 def test_decoding_context_layer(pkg, gpu, oracle, rng, causal, relu, d, H):
@@ -182,31 +210,41 @@ def test_decoding_context_layer(pkg, gpu, oracle, rng, causal, relu, d, H):
 
 
 def test_decoding_context_layer_weight_cache(pkg, gpu, oracle, rng):
-    """mgpuLLMOpsCacheWeights(1): the fp32 weights are cast once, when first seen, and later calls reuse the
-    fp16 copies - same bits as the per-call casts; switching the cache off and on again drops the copies, so
-    weights changed in place in between are picked up."""
+    """mgpuLLMOpsCacheWeights(1): the fp32 weights are cast once, when first seen (the matrices into a transposed
+    fp16 copy that a different library kernel multiplies, so the result is checked against the oracle, not against
+    the bits of the per-call path), and later calls reuse the copies; switching the cache off and on again drops
+    them, so weights changed in place in between are picked up."""
     import torch
     B, S, d, ffn, H = 2, 128, 512, 1024, 8
     f = lambda *s, sc=0.03: (sc * rng.standard_normal(s)).astype(np.float32)
-    x = to_dev(rng.standard_normal((B, S, d)).astype(np.float32), gpu)
-    W = [to_dev(w, gpu) for w in (f(d, 3 * d), f(d, d), f(d), f(d, ffn), f(ffn), f(ffn, d), f(d))]
+    x = rng.standard_normal((B, S, d)).astype(np.float32)
+    Wh = [f(d, 3 * d), f(d, d), f(d), f(d, ffn), f(ffn), f(ffn, d), f(d)]
+    xd, W = to_dev(x, gpu), [to_dev(w, gpu) for w in Wh]
     lib = pkg.ops()
-    plain = pkg.decoding_context_layer(x, *W, heads=H).clone()
+
+    def close(got, weights):
+        ref = oracle.decoding_context_layer(x, *weights, heads=H)
+        err = np.abs(got.cpu().numpy() - ref)
+        return bool(np.all(err <= layer_tol(ref))) and err.mean() <= 5e-4
+
+    plain = pkg.decoding_context_layer(xd, *W, heads=H).clone()
     lib.mgpuLLMOpsCacheWeights(1)
     try:
-        first = pkg.decoding_context_layer(x, *W, heads=H).clone()     # fills the cache
-        again = pkg.decoding_context_layer(x, *W, heads=H).clone()     # served from it
-        assert torch.equal(first, plain) and torch.equal(again, plain)
-        W[1].mul_(0.5)                                                 # in place: the cache does not see it
-        stale = pkg.decoding_context_layer(x, *W, heads=H).clone()
-        assert torch.equal(stale, plain)
+        first = pkg.decoding_context_layer(xd, *W, heads=H).clone()     # fills the cache
+        again = pkg.decoding_context_layer(xd, *W, heads=H).clone()     # served from it
+        assert close(first, Wh) and torch.equal(again, first)
+        assert (first - plain).abs().max().item() <= 2e-2               # another kernel's rounding, no more
+        W[1].mul_(0.5)                                                  # in place: the cache does not see it
+        stale = pkg.decoding_context_layer(xd, *W, heads=H).clone()
+        assert torch.equal(stale, first)
         lib.mgpuLLMOpsCacheWeights(0)
         lib.mgpuLLMOpsCacheWeights(1)
-        fresh = pkg.decoding_context_layer(x, *W, heads=H).clone()
+        fresh = pkg.decoding_context_layer(xd, *W, heads=H).clone()
     finally:
         lib.mgpuLLMOpsCacheWeights(0)
-    want = pkg.decoding_context_layer(x, *W, heads=H)
-    assert torch.equal(fresh, want) and not torch.equal(fresh, plain)
+    Wh[1] = Wh[1] * np.float32(0.5)
+    assert close(fresh, Wh) and not close(fresh, [w if i != 1 else w * np.float32(2) for i, w in enumerate(Wh)])
+    assert close(pkg.decoding_context_layer(xd, *W, heads=H), Wh)       # per-call casts again
     assert lib.mgpuOpsTakeLastError() is None
 
 
