@@ -93,6 +93,13 @@ bool weightCacheOn = false;
 struct CachedWeight {
   void *half = nullptr;
   hipEvent_t ready = nullptr; // recorded behind the conversion that filled the copy
+  bool done = false;          // the event has been seen complete: nobody needs to wait for it any more
+  // What a stream that is about to read the copy has to wait for (nothing, once the conversion
+  // has finished: a wait on a complete event still costs the stream a barrier packet).
+  hipEvent_t pending() {
+    if (!done && hipEventQuery(ready) == hipSuccess) done = true;
+    return done ? nullptr : ready;
+  }
 };
 // (array, rows, columns - 0 for a vector -, stored K-major?)
 using WeightKey = std::tuple<const void *, int64_t, int64_t, bool>;
@@ -101,7 +108,7 @@ std::map<WeightKey, CachedWeight> weightCache;
 // The cache's copy of a weight or bias array, made now - on `convert`, behind whatever that
 // stream already holds - if this is the first sight of it.  fp32 arrays are cast to fp16; a matrix
 // asked for K-major is stored transposed.  scratchMutex held; not under stream capture.
-const CachedWeight &cachedWeight(const void *src, bool srcIsF32, int64_t rows, int64_t cols, bool kMajor,
+CachedWeight &cachedWeight(const void *src, bool srcIsF32, int64_t rows, int64_t cols, bool kMajor,
                                  hipStream_t convert) {
   const WeightKey key{src, rows, cols, kMajor};
   auto hit = weightCache.find(key);
@@ -320,9 +327,9 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
       if (useCache) {
         const bool transposed = op.cols && kMajor[op.group];
         if (!weightCache.count(WeightKey{op.src, op.rows, op.cols, transposed})) fork(); // the conversion runs on the side stream
-        const CachedWeight &cw = cachedWeight(op.src, true, op.rows, op.cols, transposed, copyStream);
+        CachedWeight &cw = cachedWeight(op.src, true, op.rows, op.cols, transposed, copyStream);
         op.half = cw.half;
-        cachedReady[i] = cw.ready; // (an event long complete costs the stream nothing)
+        cachedReady[i] = cw.pending();
       } else {
         fork();
         op.half = arena.at(op.slot);
@@ -448,8 +455,8 @@ void bertEncoderLayerF16(const void *x, const void *wqkv, const void *bqkv, cons
     if (weightCacheOn && !isCapturing(stream)) {
       auto fromCache = [&](Weight &w, int64_t K, int64_t N, int act) {
         if (!gemmPrefersKMajor(DType::F16, M, N, K, true, act, false)) return;
-        const CachedWeight &cw = cachedWeight(w.w, false, K, N, true, stream);
-        MGPU_CHECK_HIP(hipStreamWaitEvent(stream, cw.ready, 0)); // (filled by a call on another stream, perhaps)
+        CachedWeight &cw = cachedWeight(w.w, false, K, N, true, stream);
+        if (hipEvent_t e = cw.pending()) MGPU_CHECK_HIP(hipStreamWaitEvent(stream, e, 0)); // (filled by another stream, perhaps)
         w = Weight{cw.half, true};
       };
       fromCache(wq, d, 3 * d, ACT_NONE);
