@@ -97,7 +97,10 @@ struct CachedWeight {
   // What a stream that is about to read the copy has to wait for (nothing, once the conversion
   // has finished: a wait on a complete event still costs the stream a barrier packet).
   hipEvent_t pending() {
-    if (!done && hipEventQuery(ready) == hipSuccess) done = true;
+    if (!done) {
+      if (hipEventQuery(ready) == hipSuccess) done = true;
+      else (void)hipGetLastError(); // "not ready" is an answer, not an error the next launch check should find
+    }
     return done ? nullptr : ready;
   }
 };
