@@ -71,6 +71,9 @@ OPS_SIGNATURES = {
     "mgpuPool2d": (None, [_c_void_p] * 2 + [_c_int64] * 15 + [_c_void_p]),
     "mgpuMatmulExF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuMatmulExBF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
+    "mgpuPackWeight16": (None, [_c_void_p] * 2 + [_c_int64] * 2 + [_c_void_p]),
+    "mgpuMatmulExPackedF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
+    "mgpuMatmulExPackedBF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuGemmMfmaF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuGemmMfmaBF16": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
     "mgpuMatmulExF32": (None, [_c_void_p] * 5 + [_c_int64] * 3 + [_c_int32] * 3 + [_c_void_p]),
@@ -349,18 +352,35 @@ def qkv_bias_transpose(qkv, bias, stream=None):
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
 
 
+def pack_weight(w, stream=None):
+    """mgpuPackWeight16: the K-major copy ([N, K]) of a 16-bit [K, N] weight, for matmul_ex(kernel="packed")."""
+    import torch
+    assert w.dtype in (torch.float16, torch.bfloat16) and w.dim() == 2 and w.is_contiguous()
+    K, N = w.shape
+    packed = torch.empty((N, K), dtype=w.dtype, device=w.device)
+    lib = ops()
+    lib.mgpuPackWeight16(_ptr(packed), _ptr(w), K, N, _stream_handle(stream))
+    _check(lib)
+    return packed
+
+
 def matmul_ex(x, w, bias=None, residual=None, act: int = ACT_NONE, stream=None, kernel: str = "auto"):
     """kernel "auto": mgpuMatmulEx*, i.e. the library or the hand-written MFMA kernel as
     the committed table and the fixed rule of the library say; "mfma": the hand-written kernel itself (fp16 / bf16, M a multiple
-    of 128, N of 128 or 96, K of 32)."""
+    of 128, N of 128 or 96, K of 32); "packed": mgpuMatmulExPacked*, w being the [N, K] copy pack_weight made."""
     import torch
     M, K = x.shape
-    K2, N = w.shape
+    if kernel == "packed":
+        N, K2 = w.shape
+    else:
+        K2, N = w.shape
     assert K == K2
     out = torch.empty((M, N), dtype=x.dtype, device=x.device)
     lib = ops()
     if kernel == "mfma":
         fn = {torch.float16: lib.mgpuGemmMfmaF16, torch.bfloat16: lib.mgpuGemmMfmaBF16}[x.dtype]
+    elif kernel == "packed":
+        fn = {torch.float16: lib.mgpuMatmulExPackedF16, torch.bfloat16: lib.mgpuMatmulExPackedBF16}[x.dtype]
     else:
         assert kernel == "auto", kernel
         fn = {torch.float16: lib.mgpuMatmulExF16, torch.bfloat16: lib.mgpuMatmulExBF16,

@@ -299,6 +299,29 @@ void mgpuMatmulExF16(void *input, void *weight, void *bias, void *output, void *
                    hasRelu, hasResidual != 0, S(stream));
   });
 }
+void mgpuPackWeight16(void *packed, void *weight, int64_t K, int64_t N, mgpuStream_t stream) {
+  guarded([&] {
+    if (K < 0 || N < 0) mgpu::fail("mgpuPackWeight16: negative shape");
+    if (packed == weight && K > 0 && N > 0) mgpu::fail("mgpuPackWeight16: packed and weight must be different arrays");
+    mgpu::transpose16(packed, weight, K, N, S(stream));
+  });
+}
+void mgpuMatmulExPackedF16(void *input, void *packedWeight, void *bias, void *output, void *residual,
+                           int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
+                           int32_t hasResidual, mgpuStream_t stream) {
+  guarded([&] {
+    mgpu::matmulEx(mgpu::DType::F16, input, packedWeight, bias, output, residual, M, N, K, hasBias != 0,
+                   hasRelu, hasResidual != 0, S(stream), true);
+  });
+}
+void mgpuMatmulExPackedBF16(void *input, void *packedWeight, void *bias, void *output, void *residual,
+                            int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t hasRelu,
+                            int32_t hasResidual, mgpuStream_t stream) {
+  guarded([&] {
+    mgpu::matmulEx(mgpu::DType::BF16, input, packedWeight, bias, output, residual, M, N, K, hasBias != 0,
+                   hasRelu, hasResidual != 0, S(stream), true);
+  });
+}
 static void gemmMfmaChecked(mgpu::DType dt, void *input, void *weight, void *bias, void *output, void *residual,
                             int64_t M, int64_t N, int64_t K, int32_t hasBias, int32_t act, int32_t hasResidual,
                             hipStream_t stream) {

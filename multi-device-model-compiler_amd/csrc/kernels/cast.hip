@@ -188,13 +188,14 @@ void transposeCastF32ToF16(void *dst, const float *src, int64_t rows, int64_t co
   transpose_cast_kernel<_Float16, float><<<grid, dim3(256), 0, stream>>>(static_cast<_Float16 *>(dst), src, rows, cols);
   MGPU_CHECK_LAUNCH("transpose_cast_kernel");
 }
-void transposeF16(void *dst, const void *src, int64_t rows, int64_t cols, hipStream_t stream) {
+void transpose16(void *dst, const void *src, int64_t rows, int64_t cols, hipStream_t stream) {
   if (rows <= 0 || cols <= 0) return;
-  if (!dst || !src) fail("transposeF16: null pointer");
+  if (!dst || !src) fail("transpose16: null pointer");
   const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
-  if ((rows + 63) / 64 > 65535) fail("transposeF16: more than 4194240 rows");
-  transpose_cast_kernel<_Float16, _Float16><<<grid, dim3(256), 0, stream>>>(static_cast<_Float16 *>(dst),
-                                                                        static_cast<const _Float16 *>(src), rows, cols);
+  if ((rows + 63) / 64 > 65535) fail("transpose16: more than 4194240 rows");
+  // as 16-bit patterns (exact through the tile's floats): fp16 and bf16 alike, NaN payloads kept
+  transpose_cast_kernel<uint16_t, uint16_t><<<grid, dim3(256), 0, stream>>>(static_cast<uint16_t *>(dst),
+                                                                        static_cast<const uint16_t *>(src), rows, cols);
   MGPU_CHECK_LAUNCH("transpose_cast_kernel");
 }
 

@@ -123,7 +123,7 @@ CachedWeight &cachedWeight(const void *src, bool srcIsF32, int64_t rows, int64_t
     MGPU_CHECK_HIP(hipEventCreateWithFlags(&fresh.ready, hipEventDisableTiming));
     if (srcIsF32 && kMajor) transposeCastF32ToF16(fresh.half, static_cast<const float *>(src), rows, cols, convert);
     else if (srcIsF32) castF32ToF16(fresh.half, static_cast<const float *>(src), elems, convert);
-    else if (kMajor) transposeF16(fresh.half, src, rows, cols, convert);
+    else if (kMajor) transpose16(fresh.half, src, rows, cols, convert);
     else fail("weight cache: nothing to convert");
     MGPU_CHECK_HIP(hipEventRecord(fresh.ready, convert));
   } catch (...) {

@@ -38,9 +38,9 @@ void castF32ToF16(void *dst, const float *src, size_t size, hipStream_t stream);
 void castF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream);
 void castF32ToBF16(void *dst, const float *src, size_t size, hipStream_t stream);
 void castBF16ToF32(float *dst, const void *src, size_t size, hipStream_t stream);
-// dst[c][r] = src[r][c] of a row-major rows x cols matrix (fp32 -> fp16 / fp16 -> fp16)
+// dst[c][r] = src[r][c] of a row-major rows x cols matrix (fp32 -> fp16; any 16-bit type, bit for bit)
 void transposeCastF32ToF16(void *dst, const float *src, int64_t rows, int64_t cols, hipStream_t stream);
-void transposeF16(void *dst, const void *src, int64_t rows, int64_t cols, hipStream_t stream);
+void transpose16(void *dst, const void *src, int64_t rows, int64_t cols, hipStream_t stream);
 void fillF16(void *dst, size_t count, float value, hipStream_t stream);
 void fillI32(int32_t *dst, size_t count, int32_t value, hipStream_t stream);
 

@@ -63,6 +63,37 @@ def test_matmul_ex_f16_epilogues(pkg, gpu, oracle, rng, M, K, N):
         assert np.all(np.abs(got - ref) <= f16_tol(ref, k_ulp)), (kw.keys(), np.abs(got - ref).max())
 
 
+@pytest.mark.parametrize("M,K,N", [(512, 768, 2304), (100, 64, 72), (33, 130, 8)])
+def test_matmul_ex_packed_weight(pkg, gpu, oracle, rng, M, K, N):
+    """mgpuPackWeight16 + mgpuMatmulExPackedF16: the weight transposed once, bit for bit (odd sizes included), and
+    every epilogue on the packed copy against the oracle, to the bound of the unpacked entry point."""
+    import torch
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    w[0, 0], w[-1, -1] = np.float16(np.nan), np.float16(6e-8)          # a NaN and a subnormal travel unchanged
+    b = rng.standard_normal(N).astype(np.float16)
+    r = rng.standard_normal((M, N)).astype(np.float16)
+    tx, tw, tb, tr = [to_dev(t, gpu) for t in (x, w, b, r)]
+    packed = pkg.pack_weight(tw)
+    assert np.array_equal(packed.cpu().numpy().view(np.uint16), np.ascontiguousarray(w.T).view(np.uint16))
+    w[0, 0] = 0
+    tw = to_dev(w, gpu)
+    packed = pkg.pack_weight(tw)
+    for kw, okw in [(dict(), dict()), (dict(bias=tb), dict(bias=b)),
+                    (dict(bias=tb, act=pkg.ACT_RELU), dict(bias=b, act=oracle.ACT_RELU)),
+                    (dict(bias=tb, act=pkg.ACT_GELU), dict(bias=b, act=oracle.ACT_GELU)),
+                    (dict(bias=tb, residual=tr), dict(bias=b, residual=r))]:
+        got = pkg.matmul_ex(tx, packed, kernel="packed", **kw).cpu().numpy().astype(np.float32)
+        ref = oracle.gemm(x, w, **okw)
+        k_ulp = 2.5 if kw.get("act") == pkg.ACT_GELU else 1.0
+        assert np.all(np.abs(got - ref) <= f16_tol(ref, k_ulp)), (kw.keys(), np.abs(got - ref).max())
+    # bf16 through the same entry points
+    xb, wb = torch.randn((64, 96), device=gpu).bfloat16(), (torch.randn((96, 40), device=gpu) / 10).bfloat16()
+    got = pkg.matmul_ex(xb, pkg.pack_weight(wb), kernel="packed").float()
+    assert torch.allclose(got, pkg.matmul_ex(xb, wb).float(), atol=4e-2, rtol=2e-2)
+    assert torch.allclose(got, xb.float() @ wb.float(), atol=4e-2, rtol=2e-2)
+
+
 def bf16_bits(t):
     import torch
     return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
