@@ -83,6 +83,8 @@ def parse_args():
                     help="total footprint of the rotating buffer sets of the cold measurements, in units of the 256 MiB "
                          "Infinity Cache")
     ap.add_argument("--no-runner", action="store_true", help="skip the end-to-end --rerun figures of the two runners")
+    ap.add_argument("--no-sdpa", action="store_true",
+                    help="skip timing torch's scaled_dot_product_attention beside the attention entries")
     ap.add_argument("--tune-gemm", action="store_true",
                     help="measure the four GEMM shapes of the BERT-base layer with the tuner of the launch-loop library (library candidates "
                          "against the hand-written kernel) and print the lines of csrc/kernels/gemm_table.inc on stderr")
@@ -736,6 +738,35 @@ def main():
         del al, bl, cl
 
     # ---------------- fused MHA -------------------------------------------------
+    def torch_sdpa_us(qkv, causal):
+        """Microseconds per call of torch.nn.functional.scaled_dot_product_attention (flash backend) on the
+        q, k, v of a packed [B, S, 3, H, D] tensor; a graph of 20 calls, the fastest of R replays.  None where this
+        torch build has no such kernel for the device."""
+        try:
+            from torch.nn.attention import sdpa_kernel, SDPBackend
+            q, k, v = [qkv[:, :, i].permute(0, 2, 1, 3).contiguous() for i in range(3)]
+            with sdpa_kernel(SDPBackend.FLASH_ATTENTION):
+                call = lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=causal)
+                for _ in range(3):
+                    call()
+                torch.cuda.synchronize()
+                graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+                with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
+                    for _ in range(20):
+                        call()
+                best = None
+                for _ in range(max(3, R)):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    graph.replay()
+                    e1.record()
+                    e1.synchronize()
+                    t = e0.elapsed_time(e1) * 1e3 / 20
+                    best = t if best is None else min(best, t)
+            return best
+        except Exception:     # no flash kernel in this build / for this device: the comparison is left out
+            return None
+
     def fmha_case(name, workload, B, S, H, masked, D=64, causal=False):
         qkv = (torch.randn((B, S, 3, H, D), device=dev, generator=gen) / 8).half()
         out = torch.empty((B, S, H * D), device=dev, dtype=torch.float16)
@@ -777,6 +808,12 @@ def main():
                  "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
         if masked or causal:
             entry["dense_flop"] = flop
+        if not masked and not args.no_sdpa:
+            # what the framework's own attention (torch SDPA, flash backend) takes on this device for the same
+            # problem, from contiguous [B, H, S, D] operands: an outside reference point, not a ceiling
+            ref_us = torch_sdpa_us(qkv, causal)
+            entry["torch_sdpa_us"] = ref_us and round(ref_us, 2)
+            entry["speedup_vs_torch_sdpa"] = ref_us and round(ref_us / us, 2)
         kernels.append(entry)
 
     if want("fmha_b32_s128"):
@@ -1026,6 +1063,8 @@ def main():
             r["cache_resident_us_per_launch"] = e["cache_resident"]["us_per_launch"]
         if "hbm_frac" in e:
             r["hbm_frac"] = e["hbm_frac"]
+        if e.get("torch_sdpa_us"):
+            r["torch_sdpa_us"] = e["torch_sdpa_us"]
         return r
     by_name = {e["name"]: e for e in kernels}
     north_star = {"layernorm_f32": star(headline), "layernorm_f16": star(by_name.get("layernorm_f16")),
@@ -1033,6 +1072,9 @@ def main():
                   "fmha_b32_s128": star(by_name.get("fmha_b32_s128")),
                   "fmha_b8_s512_masked": star(by_name.get("fmha_b8_s512_masked")),
                   "bert_layer_us": by_name["bert_layer"]["value"] if "bert_layer" in by_name else None,
+                  "bert_layer_us_with_weight_cache": by_name.get("bert_layer", {}).get("us_per_call_with_weight_cache"),
+                  "decoding_layer_us": by_name["decoding_layer"]["value"] if "decoding_layer" in by_name else None,
+                  "decoding_layer_us_with_weight_cache": by_name.get("decoding_layer", {}).get("us_per_call_with_weight_cache"),
                   "peaks": {"hbm_GBs": HBM_PEAK_GBS, "mfma_f16_TFLOPs": MFMA_F16_PEAK_TFLOPS}}
 
     result = {
