@@ -85,6 +85,8 @@ def parse_args():
     ap.add_argument("--no-runner", action="store_true", help="skip the end-to-end --rerun figures of the two runners")
     ap.add_argument("--no-sdpa", action="store_true",
                     help="skip timing torch's scaled_dot_product_attention beside the attention entries")
+    ap.add_argument("--no-torch-ref", action="store_true",
+                    help="skip timing torch's own layer_norm / add / layer composition beside the entries")
     ap.add_argument("--tune-gemm", action="store_true",
                     help="measure the four GEMM shapes of the BERT-base layer with the tuner of the launch-loop library (library candidates "
                          "against the hand-written kernel) and print the lines of csrc/kernels/gemm_table.inc on stderr")
@@ -604,6 +606,43 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
 
+    def torch_graph_us(call, ncalls):
+        """Microseconds per call of `call(i)`, i = 0..ncalls-1, captured once into a graph and replayed: what the
+        framework's own kernel for the same operation takes on this device (an outside reference point).  With one
+        call per rotating buffer set a replay meets every set as cold as the timed loops above do.  The results of
+        the captured calls are kept alive so that each call writes memory of its own.  None when torch is not asked."""
+        if args.no_torch_ref:
+            return None
+        try:
+            for i in range(min(ncalls, 3)):
+                call(i)
+            torch.cuda.synchronize()
+            graph, side, keep = torch.cuda.CUDAGraph(), torch.cuda.Stream(), []
+            with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
+                for i in range(ncalls):
+                    keep.append(call(i))
+            graph.replay()
+            torch.cuda.synchronize()
+            best = None
+            for _ in range(max(3, R)):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                graph.replay()
+                e1.record()
+                e1.synchronize()
+                t = e0.elapsed_time(e1) * 1e3 / ncalls
+                best = t if best is None else min(best, t)
+            del graph, keep
+            return best
+        except Exception:
+            return None
+
+    def with_torch(entry, us_torch):
+        if us_torch:
+            entry["torch_us"] = round(us_torch, 3)
+            entry["speedup_vs_torch"] = round(us_torch / entry.get("us_per_launch", entry["value"]), 2)
+        return entry
+
     # ---------------- headline: LayerNorm fp32 (32,128,768) -------------------
     m, n = 32 * 128, 768
     ln_bytes = 2 * m * n * 4 + 2 * n * 4
@@ -637,6 +676,7 @@ def main():
                  "many bytes in and out, same rotation")
     headline = hbm_entry("layernorm_f32", "LayerNorm fp32 (32,128,768) eps=1e-5 [configs[1]]", "f32",
                          ln_bytes, ms_cold, K, ms_warm, copy_ms * 1e3 / K if loops else None, COPY_WHAT)
+    with_torch(headline, torch_graph_us(lambda i: torch.nn.functional.layer_norm(xs[i], (n,), gamma, beta, 1e-5), nsets))
     del xs, ys, slab
 
     # ---------------- LayerNorm fp16 ------------------------------------------
@@ -664,6 +704,7 @@ def main():
         check()
         kernels.append(hbm_entry("layernorm_f16", "LayerNorm fp16 (32,128,768)", "f16",
                                  2 * m * n * 2 + 2 * n * 2, ms, K, msw, copy_ms * 1e3 / K if loops else None, COPY_WHAT))
+        with_torch(kernels[-1], torch_graph_us(lambda i: torch.nn.functional.layer_norm(xh[i], (n,), gh, bh, 1e-5), nsets))
         del xh, yh, slab
 
     # ---------------- add fp32 (3,640,640) -------------------------------------
@@ -693,6 +734,7 @@ def main():
                                  copy_ms * 1e3 / K if loops else None,
                                  "two-streams-in one-out probe (xor of two 16-byte vectors per lane, non-temporal store) "
                                  "over the same buffer sets"))
+        with_torch(kernels[-1], torch_graph_us(lambda i: torch.add(aa[i], bb[i], out=cc[i]), nsets))
         del aa, bb, cc, slab
 
     # ---------------- the same two kernels where launch latency is amortised ----
@@ -960,10 +1002,23 @@ def main():
         check()
         us = ms * 1e3 / steps
         flop = 2.0 * B * S * d * (3 * d + d + ffn + ffn) + 4.0 * B * H * S * S * 64
+        def torch_bert(i):
+            F_ = torch.nn.functional
+            wqkv, bqkv, wo, bo, g1, be1, w1, b1, w2, b2, g2, be2 = P
+            qkv_ = torch.addmm(bqkv, x.view(-1, d), wqkv).view(B, S, 3, H, d // H)
+            q_, k_, v_ = [qkv_[:, :, j].transpose(1, 2) for j in range(3)]
+            ctx = F_.scaled_dot_product_attention(q_, k_, v_).transpose(1, 2).reshape(-1, d)
+            h1 = F_.layer_norm(torch.addmm(bo, ctx, wo) + x.view(-1, d), (d,), g1, be1, 1e-5)
+            f_ = F_.gelu(torch.addmm(b1, h1, w1))
+            return F_.layer_norm(torch.addmm(b2, f_, w2) + h1, (d,), g2, be2, 1e-5)
+
+        us_torch = torch_graph_us(torch_bert, 10)
         kernels.append({"name": "bert_layer", "workload": "BERT-base encoder layer fp16 (32,128,768) [configs[4]]",
                         "dtype": "f16", "metric": "us", "value": round(us, 1), "higher_is_better": False,
                         "us_per_call_no_alloc_entry_point": us_no_alloc and round(us_no_alloc, 1),
                         "us_per_call_with_weight_cache": us_cached and round(us_cached, 1),
+                        "torch_us": us_torch and round(us_torch, 1),
+                        "speedup_vs_torch": us_torch and round(us_torch / us, 2),
                         "roofline": {"bound": "mfma", "achieved": round(flop / us / 1e6, 1),
                                      "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                      "frac": round(flop / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
@@ -997,11 +1052,32 @@ def main():
         check()
         us = ms * 1e3 / steps
         flop = 2.0 * B * S * d * (3 * d + d + 2 * ffn) + 4.0 * B * H * (d // H) * (S * (S + 1) / 2)
+
+        # the same pre-LN layer composed from torch's own operators, weights cast to fp16 beforehand (the layer the
+        # reference's PyTorch benchmark builds: benchmark/PyTorch/Models/LLM.py, TransformerEncoderLayer(2048, 16,
+        # norm_first) under a causal mask)
+        Ph = [p.half() for p in P]
+
+        def torch_dec(i):
+            F_ = torch.nn.functional
+            wqkv, wo, bo, w1, b1, w2, b2 = Ph
+            x16 = x.view(-1, d).half()
+            qkv_ = (F_.layer_norm(x16, (d,)) @ wqkv).view(B, S, 3, H, d // H)
+            q_, k_, v_ = [qkv_[:, :, j].transpose(1, 2) for j in range(3)]
+            ctx = F_.scaled_dot_product_attention(q_, k_, v_, is_causal=True).transpose(1, 2).reshape(-1, d)
+            y = x16 + torch.addmm(bo, ctx, wo)
+            f_ = torch.relu(torch.addmm(b1, F_.layer_norm(y, (d,)), w1))
+            return (y + torch.addmm(b2, f_, w2)).float()
+
+        us_torch = torch_graph_us(torch_dec, 10)
         kernels.append({"name": "decoding_layer",
                         "workload": "mgpuLLMDecodingContextLayer fp32 in/out (8,512,2048), 16 heads of 128, ffn 2048, "
                                     "causal, ReLU; fp32 weights cast to fp16 on every call, as in the reference",
                         "dtype": "f16", "metric": "us", "value": round(us, 1), "higher_is_better": False,
                         "us_per_call_with_weight_cache": round(us_cached, 1),
+                        "torch_us": us_torch and round(us_torch, 1),
+                        "speedup_vs_torch": us_torch and round(us_torch / us, 2),
+                        "speedup_vs_torch_with_weight_cache": us_torch and round(us_torch / us_cached, 2),
                         "roofline": {"bound": "mfma", "achieved": round(flop / us / 1e6, 1),
                                      "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                      "frac": round(flop / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
@@ -1063,8 +1139,9 @@ def main():
             r["cache_resident_us_per_launch"] = e["cache_resident"]["us_per_launch"]
         if "hbm_frac" in e:
             r["hbm_frac"] = e["hbm_frac"]
-        if e.get("torch_sdpa_us"):
-            r["torch_sdpa_us"] = e["torch_sdpa_us"]
+        for key in ("torch_sdpa_us", "torch_us"):
+            if e.get(key):
+                r[key] = e[key]
         return r
     by_name = {e["name"]: e for e in kernels}
     north_star = {"layernorm_f32": star(headline), "layernorm_f16": star(by_name.get("layernorm_f16")),
@@ -1073,8 +1150,10 @@ def main():
                   "fmha_b8_s512_masked": star(by_name.get("fmha_b8_s512_masked")),
                   "bert_layer_us": by_name["bert_layer"]["value"] if "bert_layer" in by_name else None,
                   "bert_layer_us_with_weight_cache": by_name.get("bert_layer", {}).get("us_per_call_with_weight_cache"),
+                  "bert_layer_torch_us": by_name.get("bert_layer", {}).get("torch_us"),
                   "decoding_layer_us": by_name["decoding_layer"]["value"] if "decoding_layer" in by_name else None,
                   "decoding_layer_us_with_weight_cache": by_name.get("decoding_layer", {}).get("us_per_call_with_weight_cache"),
+                  "decoding_layer_torch_us": by_name.get("decoding_layer", {}).get("torch_us"),
                   "peaks": {"hbm_GBs": HBM_PEAK_GBS, "mfma_f16_TFLOPs": MFMA_F16_PEAK_TFLOPS}}
 
     result = {
@@ -1088,6 +1167,7 @@ def main():
                    "buffer_sets": rotating_sets(2 * m * n * 4)},
         "repeats": R, "roofline": headline["roofline"], "cache_resident": headline.get("cache_resident"),
         "copy_ceiling": headline.get("copy_ceiling"), "frac_of_copy_ceiling": headline.get("frac_of_copy_ceiling"),
+        "torch_us": headline.get("torch_us"), "speedup_vs_torch": headline.get("speedup_vs_torch"),
         "traffic_counted_at_commit": TRAFFIC_COMMIT,
         "cpu_baseline": cpu, "ceilings": ceilings, "fmha_phases": phases, "kernels": kernels,
         "runner_end_to_end": runner,
