@@ -185,10 +185,26 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
   // of two stages, the long block first measured faster (b8 s1024 h16: 46.5
   // against 49.6 us).
   constexpr bool kCanPair = CAUSAL && D <= 128; // at 256 the second pass is compiled out
-  const bool paired = kCanPair && pairItems;
+  const bool paired = kCanPair && pairItems == 1;
   const int nItems = paired ? (nQB + 1) / 2 : nQB; // work items per (batch, head)
-  const int item = wid % nItems;
-  const int bh = wid / nItems;
+  int item = wid % nItems;
+  int bh = wid / nItems;
+  // Unpaired causal launches carry blocks of nQB different lengths.  pairItems = 2 asks for them
+  // longest first within each XCD's run: the long blocks start at once and the short ones fill in
+  // behind them, where index order gave a compute unit two blocks of the same length - two of the
+  // longest for a quarter of the units (b8 s512 h16 d128: 23.0 -> 20.7 us, b16 s512 h12 d64: 19.5 ->
+  // 14.8 us, b2 s2048 h16 d64: 41.8 -> 34.6 us).
+  if (CAUSAL && !paired && pairItems == 2 && nblk % 8 == 0 && (nblk / 8) % nQB == 0) {
+    const int nbh = nblk / 8 / nQB; // (batch, head)s of this XCD
+    const int rank = bid / 8;       // position in the XCD's dispatch order; 0 gets a longest block
+    item = nQB - 1 - rank / nbh;
+    bh = (bid % 8) * nbh + rank % nbh;
+  } else if (CAUSAL && !paired && pairItems == 2) {
+    // (batch, head)s that do not divide over the XCDs: longest first over the whole grid
+    const int nbh = nblk / nQB;
+    item = nQB - 1 - bid / nbh;
+    bh = bid % nbh;
+  }
   const int h = bh % H;
   const int b = bh / H;
 

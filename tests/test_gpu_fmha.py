@@ -85,20 +85,24 @@ def test_fmha_causal(pkg, gpu, oracle, rng, B, S, H, lens):
     assert excess(got, oracle.fmha(qkv, lens, causal=True), TOL_F16) <= 1.0
 
 
+def causal_blocks_are_paired(B, S, H, cus):
+    """The launcher's rule: exactly four query blocks per (batch, head) and a halved grid of two work items per CU."""
+    return (S + 127) // 128 == 4 and B * H * 2 >= 2 * cus
+
+
 @pytest.mark.parametrize("D,B,S,H,ragged,dtype", [
     (64, 32, 512, 12, False, "f16"),   # four query blocks per (batch, head): pairs (3, 0) and (2, 1)
-    (64, 16, 640, 16, True, "f16"),    # five: pairs (4, 0), (3, 1) and block 2 alone; ragged key counts
+    (64, 16, 500, 16, True, "f16"),    # the last block twelve rows short; ragged key counts
     (128, 32, 512, 8, False, "f16"),   # the 128-wide geometry, exactly two work items per CU
-    (128, 16, 384, 16, True, "bf16"),  # three query blocks: pair (2, 0) and block 1 alone
+    (128, 16, 450, 16, True, "bf16"),  # its last block two rows long
     (40, 32, 512, 12, True, "f16"),    # a head size padded into the 64-wide geometry
 ])
 def test_fmha_causal_paired_query_blocks(pkg, gpu, oracle, D, B, S, H, ragged, dtype):
-    """On grids that leave every CU two work items afterwards (batch x heads x ceil(query blocks / 2) >= 2 x CUs),
-    the causal kernel gives query block i and block nQB - 1 - i to one work item, which runs them one after the
+    """With four query blocks per (batch, head) on grids that leave every CU two work items afterwards, the
+    causal kernel gives query block i and block 3 - i to one work item, which runs them one after the
     other through the same LDS ring; the small problems of the other causal tests never get there."""
     import torch
-    nqb = (S + 127) // 128
-    assert B * H * ((nqb + 1) // 2) >= 2 * torch.cuda.get_device_properties(gpu).multi_processor_count
+    assert causal_blocks_are_paired(B, S, H, torch.cuda.get_device_properties(gpu).multi_processor_count)
     rng = np.random.Generator(np.random.PCG64(D * 1000 + S))
     tq = torch.from_numpy(rng.standard_normal((B, S, 3, H, D)).astype(np.float32)).to(gpu)
     tq = tq.to(torch.float16 if dtype == "f16" else torch.bfloat16)
@@ -110,6 +114,43 @@ def test_fmha_causal_paired_query_blocks(pkg, gpu, oracle, D, B, S, H, ragged, d
     got = pkg.fused_mha(tq, to_dev(lens, gpu) if ragged else None, causal=True).float().cpu().numpy()
     ref = oracle.fmha(bits.view(np.float16) if dtype == "f16" else bits, lens, causal=True, bf16=dtype == "bf16")
     assert excess(got, ref, TOL_F16 if dtype == "f16" else TOL_BF16) <= 1.0
+
+
+@pytest.mark.parametrize("D,B,S,H,ragged,packed", [
+    (64, 8, 640, 8, True, False),     # five query blocks per (batch, head), 320 blocks: 40 per XCD, longest first
+    (128, 8, 512, 16, False, False),  # the reference layer's attention at (8,512,2048): 512 blocks, two per CU
+    (64, 16, 640, 16, True, False),   # 1280 blocks: several rounds; ragged key counts
+    (128, 16, 384, 16, True, False),  # three query blocks, 128-wide heads
+    (64, 16, 300, 8, False, True),    # packed rows of unequal length under the same order
+    (64, 5, 640, 12, False, False),   # 300 blocks, not a multiple of 8: longest first over the whole grid
+    (64, 4, 768, 11, False, False),   # 264 blocks, 33 per XCD, not whole (batch, head)s: the same
+])
+def test_fmha_causal_longest_block_first(pkg, gpu, oracle, D, B, S, H, ragged, packed):
+    """Causal grids with more blocks than CUs that are not paired: the launcher has the kernel hand out each XCD's
+    query blocks longest first (another map from block id to (batch, head, query block)); every row of every
+    block must still come out."""
+    import torch
+    cus = torch.cuda.get_device_properties(gpu).multi_processor_count
+    assert cus < B * H * ((S + 127) // 128) and not causal_blocks_are_paired(B, S, H, cus)
+    rng = np.random.Generator(np.random.PCG64(D * 977 + S + B))
+    if packed:
+        lens = rng.integers(1, S + 1, B)
+        lens[:3] = [S, 1, 129]
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        tq = torch.from_numpy(rng.standard_normal((int(cu[-1]), 3, H, D)).astype(np.float32)).to(gpu).half()
+        got = pkg.fused_mha_cu_seqlens(tq, to_dev(cu, gpu), S, causal=True).float().cpu().numpy()
+        bits = tq.view(torch.int16).cpu().numpy().view(np.uint16)
+        for b in range(B):
+            ref = oracle.fmha(bits[cu[b]:cu[b + 1]][None].view(np.float16), causal=True)[0]
+            assert excess(got[cu[b]:cu[b + 1]], ref, TOL_F16) <= 1.0, f"sequence {b} of {lens[b]} rows"
+        return
+    qkv = rng.standard_normal((B, S, 3, H, D)).astype(np.float16)
+    lens = None
+    if ragged:
+        lens = rng.integers(0, S + 1, B).astype(np.int32)
+        lens[0], lens[1] = S, 1
+    got = run(pkg, gpu, qkv, lens, causal=True)
+    assert excess(got, oracle.fmha(qkv, lens, causal=True), TOL_F16) <= 1.0
 
 
 def test_fmha_causal_paired_query_blocks_over_packed_rows(pkg, gpu, oracle):
@@ -423,8 +464,8 @@ def test_fmha_profile_entry_point_matches_the_product_kernel(pkg, gpu):
     (160, 2, 64, 2, None, False, "bf16"),
     (136, 1, 65, 1, None, False, "f16"),        # the first size past the 128-wide geometry
     (248, 1, 129, 2, [129], True, "f16"),       # one chunk short of the 256-wide geometry
-    (80, 16, 384, 22, None, True, "f16"),       # 704 causal work items: query blocks in pairs, head size 80 inside 128
-    (96, 32, 300, 8, None, True, "bf16"),       # 512 paired items with a middle block (3 query blocks), ragged last tile
+    (80, 16, 512, 16, None, True, "f16"),       # 512 causal work items of two query blocks each, head size 80 inside 128
+    (96, 32, 300, 8, None, True, "bf16"),       # 768 causal blocks handed out longest first, ragged last tile
 ])
 def test_fmha_other_head_sizes(pkg, gpu, oracle, rng, D, B, S, H, lens, causal, dtype):
     """Head sizes between the tile geometries (64, 128, 256) run inside the next larger one: rows in
