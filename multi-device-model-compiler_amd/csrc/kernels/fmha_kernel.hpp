@@ -205,6 +205,18 @@ __global__ __launch_bounds__(256, (CAUSAL && D == 64) ? 3 : 2) void fmha_fwd_ker
     item = nQB - 1 - bid / nbh;
     bh = bid % nbh;
   }
+  // Sequences of unequal length: a contiguous run of (batch, head)s per XCD is a few whole
+  // sequences per XCD (one, at b8 h16), and the XCD that drew the longest sets the launch's
+  // time.  Dealing the (batch, head)s round-robin instead gives every XCD some heads of every
+  // sequence; the query blocks of one (batch, head) still share an XCD (b8 s512 h16 d128, key
+  // counts 256..512: 23.0 -> 20.6 us; b64 s512 h12 d64, 1..512: 53.5 -> 49.3).  Not with one query
+  // block per (batch, head): there the finer interleave of the rows over the XCDs costs more
+  // than the balance gains (b32 s128 h12: 6.36 -> 6.53 us).
+  if ((seqlens || cuSeqlens) && nQB >= 2 && nblk % 8 == 0 && (nblk / nItems) % 8 == 0 &&
+      !(CAUSAL && !paired && pairItems == 2 && (nblk / 8) % nQB != 0)) {
+    const int perXcd = nblk / nItems / 8;
+    bh = (bh % perXcd) * 8 + bh / perXcd;
+  }
   const int h = bh % H;
   const int b = bh / H;
 
