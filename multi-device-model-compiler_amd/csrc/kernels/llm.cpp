@@ -20,8 +20,9 @@
 //    capture, so the graph owns its temporaries and a later eager call that
 //    grows (frees and replaces) the stream's arena cannot pull memory from
 //    under a graph that is still replayed;
-//  * the side stream casts all the weights as soon as the call starts, one
-//    event per GEMM, while the input cast and the first LayerNorm run on the
+//  * the side stream casts all the weights as soon as the call starts (one
+//    event behind the first GEMM's weight, one behind the rest), while the
+//    input cast and the first LayerNorm run on the
 //    caller's stream (the reference interleaves cast and wait per GEMM, input
 //    cast included, so the first GEMM starts two casts late); the gamma = 1 /
 //    beta = 0 vectors are written once per model width, not per call;
@@ -339,13 +340,17 @@ void decodingContextLayer(float *input, float *qkv, float *gemm_weight, float *g
         castF32ToF16(op.half, op.src, op.elems(), copyStream);
         sideWork[op.group] = true;
       }
-      // the casts go out in the order the GEMMs run; a group's event sits right behind its last cast
-      if ((i == 6 || ops[i + 1].group != op.group) && sideWork[op.group])
-        MGPU_CHECK_HIP(hipEventRecord(copyEvent[op.group], copyStream));
+      // The casts go out in the order the GEMMs run.  Two events: one right behind the first GEMM's
+      // weight, one behind everything else - the later casts are long done when the second GEMM
+      // starts (they run under the first, the longest), and every wait the caller's stream does
+      // not make is a barrier packet it does not stall on.
+      if ((i == 0 || i == 6) && sideWork[op.group])
+        MGPU_CHECK_HIP(hipEventRecord(copyEvent[i == 0 ? 0 : 1], copyStream));
     }
   }
   auto join = [&](int group) {
-    if (sideWork[group]) MGPU_CHECK_HIP(hipStreamWaitEvent(stream, copyEvent[group], 0));
+    if (group <= 1 && (sideWork[group] || (group == 1 && (sideWork[2] || sideWork[3]))))
+      MGPU_CHECK_HIP(hipStreamWaitEvent(stream, copyEvent[group], 0));
     for (int i = 0; i < 7; i++)
       if (ops[i].group == group && cachedReady[i]) MGPU_CHECK_HIP(hipStreamWaitEvent(stream, cachedReady[i], 0));
   };
