@@ -153,6 +153,40 @@ def test_fmha_causal_longest_block_first(pkg, gpu, oracle, D, B, S, H, ragged, p
     assert excess(got, oracle.fmha(qkv, lens, causal=True), TOL_F16) <= 1.0
 
 
+def test_fmha_seeded_sweep_over_the_block_orders(pkg, gpu, oracle):
+    """A seeded draw of shapes, masks and length forms: whatever order the launcher hands the blocks out in (index
+    order, pairs, longest first, (batch, head)s dealt over the XCDs, packed rows), every output row is the
+    attention of its own query over its own keys."""
+    import random
+    import torch
+    rnd = random.Random(20250)
+    cases = 0
+    while cases < 14:
+        D = rnd.choice([64, 64, 128, 40])
+        H, B = rnd.choice([1, 3, 4, 8, 12, 16]), rnd.choice([1, 2, 5, 8, 16])
+        S = rnd.choice([64, 200, 256, 384, 512, 640])
+        if B * H * S * S * D > 1.2e9:
+            continue
+        causal, mode = rnd.random() < 0.5, rnd.choice(["dense", "seqlens", "cu"])
+        rng = np.random.Generator(np.random.PCG64(1000 + cases))
+        cases += 1
+        if mode == "cu":
+            lens = np.array([rnd.randint(0, S) for _ in range(B)])
+            lens[0] = S
+            cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+            qkv = rng.standard_normal((int(cu[-1]), 3, H, D)).astype(np.float16)
+            got = pkg.fused_mha_cu_seqlens(to_dev(qkv, gpu), to_dev(cu, gpu), S, causal=causal).float().cpu().numpy()
+            for b in range(B):
+                if lens[b]:
+                    ref = oracle.fmha(qkv[cu[b]:cu[b + 1]][None], causal=causal)[0]
+                    assert excess(got[cu[b]:cu[b + 1]], ref, TOL_F16) <= 1.0, (D, B, S, H, causal, mode, b)
+        else:
+            qkv = rng.standard_normal((B, S, 3, H, D)).astype(np.float16)
+            lens = np.array([rnd.randint(0, S) for _ in range(B)], np.int32) if mode == "seqlens" else None
+            got = run(pkg, gpu, qkv, lens, causal=causal)
+            assert excess(got, oracle.fmha(qkv, lens, causal=causal), TOL_F16) <= 1.0, (D, B, S, H, causal, mode)
+
+
 def test_fmha_causal_paired_query_blocks_over_packed_rows(pkg, gpu, oracle):
     """The same pairing with the sequences given as prefix sums over packed rows: a pair's late block may lie
     wholly beyond a short sequence while its early block does not."""
