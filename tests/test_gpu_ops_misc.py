@@ -193,6 +193,32 @@ def test_bert_encoder_layer_config4(pkg, gpu, oracle):
         assert err.mean() <= 5e-4
 
 
+def test_weight_cache_shared_by_two_streams(pkg, gpu, rng):
+    """The cache is per process, not per stream: a call on one stream fills it (the conversions run on that stream's
+    side stream) and a call issued right behind it on another stream, before anything has finished, must wait
+    for those conversions - both give the result of a call made after everything has drained."""
+    import torch
+    B, S, d, ffn, H = 4, 256, 1024, 1024, 8
+    f = lambda *s, sc=0.03: to_dev((sc * rng.standard_normal(s)).astype(np.float32), gpu)
+    x = to_dev(rng.standard_normal((B, S, d)).astype(np.float32), gpu)
+    lib = pkg.ops()
+    for trial in range(3):
+        W = [f(d, 3 * d), f(d, d), f(d), f(d, ffn), f(ffn), f(ffn, d), f(d)]   # new arrays: the cache has not seen them
+        s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+        torch.cuda.synchronize()
+        lib.mgpuLLMOpsCacheWeights(1)
+        try:
+            a = pkg.decoding_context_layer(x, *W, heads=H, stream=s1)
+            b = pkg.decoding_context_layer(x, *W, heads=H, stream=s2)
+            torch.cuda.synchronize()
+            settled = pkg.decoding_context_layer(x, *W, heads=H)
+            torch.cuda.synchronize()
+        finally:
+            lib.mgpuLLMOpsCacheWeights(0)
+        assert torch.equal(a, settled) and torch.equal(b, settled), trial
+    assert lib.mgpuOpsTakeLastError() is None
+
+
 def test_bert_encoder_layer_weight_cache(pkg, gpu, oracle):
     """With mgpuLLMOpsCacheWeights(1) the BERT layer hands the GEMMs the committed table marks (QKV and FFN2 at
     configs[4]) a transposed copy of their weight, kept by the cache: same layer against the oracle, the same
